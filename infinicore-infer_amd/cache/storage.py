@@ -1,0 +1,51 @@
+"""Device memory of the cache: the page planes of each group and the
+per-request state tensors.
+
+Layout of one cache slot (one attention layer's keys or values):
+``[num_pages, n_kv_heads, page_size, head_dim]``: the keys of one head inside a
+page are one contiguous run, which is what the attention kernels stream.
+A group holds ``[n_slots, 2 (K, V), num_pages, n_kv_heads, page_size, head_dim]``.
+"""
+from typing import Dict, List, Sequence, Tuple
+
+import torch
+
+from .manager import GroupSpec
+
+
+class CacheStorage:
+    def __init__(self, groups: Sequence[GroupSpec], num_pages: Sequence[int], page_size: int,
+                 dtype: torch.dtype, device):
+        self.page_size = page_size
+        self.dtype = dtype
+        self.device = device
+        self.group_planes: List[torch.Tensor] = []
+        self._slot_index: Dict[int, Tuple[int, int]] = {}      # cache slot -> (group, index in group)
+        for g, spec in enumerate(groups):
+            planes = torch.empty((len(spec.slots), 2, num_pages[g], spec.n_kv_heads, page_size, spec.head_dim),
+                                 dtype=dtype, device=device)
+            self.group_planes.append(planes)
+            for i, s in enumerate(spec.slots):
+                self._slot_index[s] = (g, i)
+        self.state: Dict[int, torch.Tensor] = {}               # cache slot -> [max_requests, ...]
+
+    def add_state(self, slot: int, max_requests: int, shape, dtype) -> torch.Tensor:
+        t = torch.zeros((max_requests,) + tuple(shape), dtype=dtype, device=self.device)
+        self.state[slot] = t
+        return t
+
+    def group_of(self, slot: int) -> int:
+        return self._slot_index[slot][0]
+
+    def kv(self, slot: int):
+        """(K plane, V plane) of a cache slot."""
+        g, i = self._slot_index[slot]
+        return self.group_planes[g][i, 0], self.group_planes[g][i, 1]
+
+    def zero_state(self, state_slot: int) -> None:
+        for t in self.state.values():
+            t[state_slot].zero_()
+
+    def bytes(self) -> int:
+        n = sum(p.numel() * p.element_size() for p in self.group_planes)
+        return n + sum(t.numel() * t.element_size() for t in self.state.values())

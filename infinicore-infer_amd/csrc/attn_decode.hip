@@ -1,0 +1,264 @@
+// Attention of single new tokens over the paged cache (decoding), split over
+// the keys so that few requests still fill the chip.
+//
+// Pass 1, grid (splits, kv heads, tokens), 256 threads: a block streams its
+// share of one request's keys and values of one kv head once and serves the
+// query heads of that group, four at a time.  DH/VEC lanes share a key
+// (VEC = 16 bytes of elements per lane), so a wave reads whole contiguous
+// rows; every lane keeps a float32 running softmax for its keys, which are
+// merged across the lane groups, the four waves, and (pass 2) the splits.
+// Pass 2, grid (tokens * heads): combines the splits and writes the output.
+//
+// Cache layout of one layer: K and V planes [num_pages, n_kv_heads, page_size, head_dim].
+#include "common.h"
+
+constexpr int kDecThreads = 256;
+constexpr int kDecWaves = kDecThreads / 64;
+constexpr int kDecUnroll = 4;
+
+template <typename T> struct Vec16;
+template <> struct Vec16<float> {
+    static constexpr int N = 4;
+    __device__ static void load(const float* p, float* o) {
+        const float4 v = *reinterpret_cast<const float4*>(p);
+        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    }
+};
+template <> struct Vec16<bf16> {
+    static constexpr int N = 8;
+    __device__ static void load(const bf16* p, float* o) {
+        const uint4 v = *reinterpret_cast<const uint4*>(p);
+        o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+        o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+        o[4] = __uint_as_float(v.z << 16); o[5] = __uint_as_float(v.z & 0xffff0000u);
+        o[6] = __uint_as_float(v.w << 16); o[7] = __uint_as_float(v.w & 0xffff0000u);
+    }
+};
+
+// merge running-softmax state b into a
+__device__ __forceinline__ void merge_state(float& m, float& l, float* acc, int n,
+                                            float mb, float lb, const float* accb) {
+    const float mn = fmaxf(m, mb);
+    if (mn == -INFINITY) return;                 // both empty
+    const float ca = expf(m - mn), cb = expf(mb - mn);
+    l = l * ca + lb * cb;
+    for (int i = 0; i < n; ++i) acc[i] = acc[i] * ca + accb[i] * cb;
+    m = mn;
+}
+
+template <typename T, int DH, int GQ>
+__global__ void __launch_bounds__(kDecThreads)
+attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
+                         const T* __restrict__ kcache, const T* __restrict__ vcache,
+                         const int* __restrict__ block_tables, int bt_stride,
+                         const int* __restrict__ tok_list, const int* __restrict__ token_req,
+                         const int* __restrict__ positions,
+                         float* __restrict__ part_acc, float* __restrict__ part_ml,
+                         int nh, int nkvh, int page_size, float scale, int window, int nsplit) {
+    constexpr int VEC = Vec16<T>::N;
+    constexpr int LPK = DH / VEC;                 // lanes per key
+    constexpr int KPW = 64 / LPK;                 // keys per wave per step
+    constexpr int KPB = KPW * kDecWaves;          // keys per block per step
+    static_assert(DH % VEC == 0 && 64 % LPK == 0, "head size must split a wave evenly");
+
+    __shared__ float sm_acc[kDecWaves][GQ][DH];
+    __shared__ float sm_ml[kDecWaves][GQ][2];
+
+    const int split = blockIdx.x, kvh = blockIdx.y, n = blockIdx.z;
+    const int t = tok_list ? tok_list[n] : n;
+    const int g = nh / nkvh;
+    const int pos = positions[t];
+    const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
+    const int lo0 = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int nkeys = pos + 1 - lo0;
+    const int per = (nkeys + nsplit - 1) / nsplit;
+    const int lo = lo0 + split * per;
+    int hi = lo + per;
+    if (hi > pos + 1) hi = pos + 1;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int sub = lane % LPK;                   // which 16-byte slice of the row
+    const int grp = lane / LPK;                   // which key of the wave's step
+    const size_t head_stride = (size_t)page_size * DH;
+
+    for (int h0 = 0; h0 < g; h0 += GQ) {
+        float qv[GQ][VEC], acc[GQ][VEC], m[GQ], l[GQ];
+#pragma unroll
+        for (int j = 0; j < GQ; ++j) {
+            m[j] = -INFINITY; l[j] = 0.f;
+            const int hh = (h0 + j < g) ? h0 + j : g - 1;
+            Vec16<T>::load(q + (size_t)t * q_stride + (size_t)(kvh * g + hh) * DH + sub * VEC, qv[j]);
+#pragma unroll
+            for (int i = 0; i < VEC; ++i) { qv[j][i] *= scale; acc[j][i] = 0.f; }
+        }
+
+        for (int kb = lo + wave * KPW + grp; kb < hi; kb += kDecUnroll * KPB) {
+            float kf[kDecUnroll][VEC], vf[kDecUnroll][VEC];
+            bool ok[kDecUnroll];
+#pragma unroll
+            for (int u = 0; u < kDecUnroll; ++u) {
+                const int key = kb + u * KPB;
+                ok[u] = key < hi;
+                if (ok[u]) {
+                    const int pg = bt[key / page_size];
+                    const int off = key % page_size;
+                    const size_t base = ((size_t)pg * nkvh + kvh) * head_stride + (size_t)off * DH + sub * VEC;
+                    Vec16<T>::load(kcache + base, kf[u]);
+                    Vec16<T>::load(vcache + base, vf[u]);
+                }
+            }
+#pragma unroll
+            for (int j = 0; j < GQ; ++j) {
+                float s[kDecUnroll];
+                float mx = m[j];
+#pragma unroll
+                for (int u = 0; u < kDecUnroll; ++u) {
+                    float d = 0.f;
+                    if (ok[u]) {
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) d += qv[j][i] * kf[u][i];
+                    }
+#pragma unroll
+                    for (int o = LPK >> 1; o > 0; o >>= 1) d += __shfl_xor(d, o, kWave);
+                    s[u] = ok[u] ? d : -INFINITY;
+                    mx = fmaxf(mx, s[u]);
+                }
+                if (mx == -INFINITY) continue;     // this lane group has seen no key yet
+                const float corr = expf(m[j] - mx);
+                float lsum = l[j] * corr;
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) acc[j][i] *= corr;
+#pragma unroll
+                for (int u = 0; u < kDecUnroll; ++u) {
+                    if (ok[u]) {
+                        const float p = expf(s[u] - mx);
+                        lsum += p;
+#pragma unroll
+                        for (int i = 0; i < VEC; ++i) acc[j][i] += p * vf[u][i];
+                    }
+                }
+                l[j] = lsum;
+                m[j] = mx;
+            }
+        }
+
+        // merge the lane groups of the wave (lanes with the same `sub`)
+#pragma unroll
+        for (int j = 0; j < GQ; ++j) {
+#pragma unroll
+            for (int o = LPK; o < 64; o <<= 1) {
+                const float mb = __shfl_xor(m[j], o, kWave);
+                const float lb = __shfl_xor(l[j], o, kWave);
+                float ab[VEC];
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) ab[i] = __shfl_xor(acc[j][i], o, kWave);
+                merge_state(m[j], l[j], acc[j], VEC, mb, lb, ab);
+            }
+        }
+        __syncthreads();                            // LDS free from the previous head chunk
+        if (grp == 0) {
+#pragma unroll
+            for (int j = 0; j < GQ; ++j) {
+#pragma unroll
+                for (int i = 0; i < VEC; ++i) sm_acc[wave][j][sub * VEC + i] = acc[j][i];
+                if (sub == 0) { sm_ml[wave][j][0] = m[j]; sm_ml[wave][j][1] = l[j]; }
+            }
+        }
+        __syncthreads();
+        // merge the waves: thread (j, d) for j < GQ, d < DH
+        for (int idx = threadIdx.x; idx < GQ * DH; idx += kDecThreads) {
+            const int j = idx / DH, d = idx - j * DH;
+            if (h0 + j >= g) continue;
+            float mm = -INFINITY;
+            for (int w = 0; w < kDecWaves; ++w) mm = fmaxf(mm, sm_ml[w][j][0]);
+            float a = 0.f, ll = 0.f;
+            if (mm != -INFINITY) {
+                for (int w = 0; w < kDecWaves; ++w) {
+                    const float c = expf(sm_ml[w][j][0] - mm);
+                    a += sm_acc[w][j][d] * c;
+                    ll += sm_ml[w][j][1] * c;
+                }
+            }
+            const int h = kvh * g + h0 + j;
+            const size_t pidx = ((size_t)n * nh + h) * nsplit + split;
+            part_acc[pidx * DH + d] = a;
+            if (d == 0) { part_ml[pidx * 2] = mm; part_ml[pidx * 2 + 1] = ll; }
+        }
+    }
+}
+
+template <typename T>
+__global__ void attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                                          const int* __restrict__ tok_list, T* __restrict__ out,
+                                          int out_stride, int nh, int dh, int nsplit) {
+    const int n = blockIdx.x / nh, h = blockIdx.x % nh;
+    const int t = tok_list ? tok_list[n] : n;
+    const size_t base = ((size_t)n * nh + h) * nsplit;
+    float mm = -INFINITY;
+    for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
+    float ll = 0.f;
+    for (int s = 0; s < nsplit; ++s) {
+        const float ms = part_ml[(base + s) * 2];
+        if (ms != -INFINITY) ll += part_ml[(base + s) * 2 + 1] * expf(ms - mm);
+    }
+    const float inv = 1.0f / ll;
+    for (int d = threadIdx.x; d < dh; d += blockDim.x) {
+        float a = 0.f;
+        for (int s = 0; s < nsplit; ++s) {
+            const float ms = part_ml[(base + s) * 2];
+            if (ms != -INFINITY) a += part_acc[(base + s) * dh + d] * expf(ms - mm);
+        }
+        out[(size_t)t * out_stride + (size_t)h * dh + d] = from_f32<T>(a * inv);
+    }
+}
+
+template <typename T, int DH>
+static int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
+                         const void* vcache, const int* block_tables, int bt_stride, const int* tok_list,
+                         const int* token_req, const int* positions, float* part_acc, float* part_ml,
+                         int n_tok, int nh, int nkvh, int page_size, float scale, int window, int nsplit,
+                         hipStream_t stream) {
+    dim3 grid(nsplit, nkvh, n_tok), block(kDecThreads);
+    if (nh == nkvh)
+        hipLaunchKernelGGL((attn_decode_split_kernel<T, DH, 1>), grid, block, 0, stream, (const T*)q, q_stride,
+                           (const T*)kcache, (const T*)vcache, block_tables, bt_stride, tok_list, token_req,
+                           positions, part_acc, part_ml, nh, nkvh, page_size, scale, window, nsplit);
+    else
+        hipLaunchKernelGGL((attn_decode_split_kernel<T, DH, 4>), grid, block, 0, stream, (const T*)q, q_stride,
+                           (const T*)kcache, (const T*)vcache, block_tables, bt_stride, tok_list, token_req,
+                           positions, part_acc, part_ml, nh, nkvh, page_size, scale, window, nsplit);
+    int st = ic_launch_status();
+    if (st) return st;
+    hipLaunchKernelGGL(attn_decode_reduce_kernel<T>, dim3(n_tok * nh), dim3(64), 0, stream, part_acc, part_ml,
+                       tok_list, (T*)out, out_stride, nh, DH, nsplit);
+    return ic_launch_status();
+}
+
+// Head sizes with a tiled decode kernel.
+IC_EXPORT int ic_attn_decode_supported(int dtype, int dh) {
+    return (dtype == IC_F32 || dtype == IC_BF16) && (dh == 64 || dh == 128);
+}
+
+// part_acc: float32 [n_tok, nh, nsplit, dh]; part_ml: float32 [n_tok, nh, nsplit, 2].
+// tok_list: rows of q/out that are decoded (nullptr: rows 0..n_tok-1).
+IC_EXPORT int ic_attn_decode(const void* q, int q_stride, void* out, int out_stride, int dtype,
+                             const void* kcache, const void* vcache, const int* block_tables,
+                             int bt_stride, const int* tok_list, const int* token_req,
+                             const int* positions, float* part_acc, float* part_ml, int n_tok, int nh,
+                             int nkvh, int dh, int page_size, float scale, int window, int nsplit,
+                             hipStream_t stream) {
+    if (n_tok <= 0) return IC_OK;
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || nsplit <= 0) return IC_ERR_ARG;
+    if (nkvh > 65535 || n_tok > 65535) return IC_ERR_ARG;
+    if (q_stride % 8 || ((uintptr_t)q & 15) || ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15)) return IC_ERR_ARG;
+#define IC_DECODE_CASE(TT, DD)                                                                          \
+    return launch_decode<TT, DD>(q, q_stride, out, out_stride, kcache, vcache, block_tables, bt_stride, \
+                                 tok_list, token_req, positions, part_acc, part_ml, n_tok, nh, nkvh,   \
+                                 page_size, scale, window, nsplit, stream)
+    if (dtype == IC_F32 && dh == 64) IC_DECODE_CASE(float, 64);
+    if (dtype == IC_F32 && dh == 128) IC_DECODE_CASE(float, 128);
+    if (dtype == IC_BF16 && dh == 64) IC_DECODE_CASE(bf16, 64);
+    if (dtype == IC_BF16 && dh == 128) IC_DECODE_CASE(bf16, 128);
+#undef IC_DECODE_CASE
+    return IC_ERR_UNSUPPORTED;
+}

@@ -1,0 +1,96 @@
+"""What one step hands to the parts: the batch as flat arrays, the cache views
+and the workspace.
+
+A batch is a list of (request, its next tokens).  Tokens are concatenated in
+entry order, as the reference does (src/models/jiuge/jiuge.cpp:147-154):
+``positions[t] = req_pos[r] + i``.  All integer arrays of a step are packed
+into one pinned host buffer and reach the device in one copy.
+"""
+from dataclasses import dataclass
+from typing import Dict, List, Optional
+
+import torch
+
+
+class Workspace:
+    """Named scratch buffers that grow to the largest size asked for and are then
+    reused, so steps of a steady shape allocate nothing and pointers stay put."""
+
+    def __init__(self, device):
+        self.device = device
+        self._bufs: Dict[str, torch.Tensor] = {}
+
+    def buffer(self, name: str, shape, dtype) -> torch.Tensor:
+        n = 1
+        for s in shape:
+            n *= int(s)
+        key = "%s/%s" % (name, str(dtype))
+        buf = self._bufs.get(key)
+        if buf is None or buf.numel() < n:
+            buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        return buf[:n].view(*shape)
+
+    def bytes(self) -> int:
+        return sum(b.numel() * b.element_size() for b in self._bufs.values())
+
+
+@dataclass
+class LayerCacheView:
+    """What a mixer sees of its cache slot in this step."""
+    k: Optional[torch.Tensor] = None             # [pages, kv_heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None
+    slots: Optional[torch.Tensor] = None         # int32 [T]: token slot of each new token in this group
+    block_tables: Optional[torch.Tensor] = None  # int32 [R, max_blocks]
+    state: Optional[torch.Tensor] = None         # [max_requests, ...] fixed-size state of this slot
+    writes: bool = True
+
+
+class StepContext:
+    """Flat description of a step's batch.  Built by ``Engine``; read by parts."""
+
+    def __init__(self):
+        self.T = 0                       # tokens in the step
+        self.R = 0                       # requests in the step
+        self.page_size = 0
+        self.ws: Workspace = None
+        # device arrays
+        self.tokens = None               # int32 [T]
+        self.positions = None            # int32 [T]
+        self.token_req = None            # int32 [T]  batch row of each token
+        self.state_slots = None          # int32 [R]  state slot of each request
+        self.want_rows = None            # int32 [W]  token rows whose logits are wanted
+        self.n_want = 0
+        self.decode_rows = None          # int32 [n_decode_rows] rows that are a request's single token
+        self.n_decode_rows = 0
+        self.decode_rows_identity = False
+        self.prefill_tiles = None        # int32 [n_tiles, 4] (batch row, first token row, rows, first position)
+        self.n_prefill_tiles = 0
+        # host copies
+        self.req_start: List[int] = []   # first token row of each request (R + 1 entries)
+        self.req_pos: List[int] = []     # position of each request's first new token
+        self.req_len: List[int] = []
+        self.req_ids: List[object] = []
+        self.host_state_slots: List[int] = []
+        self.max_position = 0            # largest position in the step
+        self.max_context = 0             # most keys any single-token row sees
+        self.cu_count = 256              # compute units, for split heuristics
+        self.fixed_decode_splits: Optional[int] = None
+        self._views: Dict[int, LayerCacheView] = {}
+
+    def cache_view(self, entry) -> LayerCacheView:
+        v = self._views[entry.cache]
+        if v.writes != entry.writes_cache:
+            v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache)
+        return v
+
+    def decode_splits(self, n_kv_heads: int, window: int = 0) -> int:
+        """How many ways to split the keys of single-token rows so that the grid
+        fills the chip: enough blocks for ~4 per compute unit, at least 256 keys each."""
+        if self.fixed_decode_splits is not None:
+            return self.fixed_decode_splits
+        keys = self.max_context if not window else min(self.max_context, window)
+        blocks = max(1, self.n_decode_rows * n_kv_heads)
+        want = max(1, (4 * self.cu_count + blocks - 1) // blocks)
+        most = max(1, keys // 256)
+        return int(max(1, min(want, most, 64)))

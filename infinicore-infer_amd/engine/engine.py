@@ -1,0 +1,292 @@
+"""The step function: a batch of (request, its next tokens) runs as one batch
+from the cache and returns the logits at the wanted places.
+
+The reference's step is inferBatch / forwardBatch
+(include/infinicore_infer/models/jiuge.h:89-110, src/models/jiuge/jiuge.cpp:114-298):
+tokens of all requests concatenated, req_lens, req_pos and one cache handle per
+request.  Here the cache handle is a request id known to the cache manager;
+portions of prompts and single decoded tokens may be mixed and cut anywhere.
+"""
+from dataclasses import dataclass, field
+from typing import Dict, List, Optional, Sequence
+
+import torch
+
+from ..cache import CacheManager, CacheStorage, GroupSpec, OutOfPages
+from ..config import config_from_dir
+from ..kernels import ops
+from ..parts import Runtime, build_model
+from .context import LayerCacheView, StepContext, Workspace
+
+
+@dataclass
+class StepEntry:
+    """One request's share of a step: its next tokens and the places among them
+    whose logits are wanted (indices into ``tokens``; may be empty)."""
+    req_id: object
+    tokens: Sequence[int]
+    want: Sequence[int] = field(default_factory=list)
+
+
+def _align4(n: int) -> int:
+    return (n + 3) & ~3
+
+
+class _PinnedRing:
+    """A few pinned host buffers used in turn, each guarded by an event, so a
+    buffer is not rewritten while its copy to the device may still run."""
+
+    def __init__(self, n: int = 4):
+        self.bufs = [None] * n
+        self.events = [None] * n
+        self.i = 0
+
+    def get(self, numel: int) -> torch.Tensor:
+        self.i = (self.i + 1) % len(self.bufs)
+        if self.events[self.i] is not None:
+            self.events[self.i].synchronize()
+        b = self.bufs[self.i]
+        if b is None or b.numel() < numel:
+            b = torch.empty(max(numel, 1024), dtype=torch.int32, pin_memory=True)
+            self.bufs[self.i] = b
+        return b
+
+    def mark(self):
+        ev = self.events[self.i]
+        if ev is None:
+            ev = torch.cuda.Event()
+            self.events[self.i] = ev
+        ev.record()
+
+
+class Engine:
+    def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 64,
+                 num_pages: Optional[int] = None):
+        """``max_tokens``: the most tokens live requests hold at any time, each
+        request's count rounded up to whole pages; every group's pool is sized for it."""
+        self.model = model
+        self.runtime: Runtime = model.runtime
+        self.device = torch.device(self.runtime.device)
+        if self.device.type != "cuda":
+            raise RuntimeError("the engine runs on the GPU only (device %s given); there is no CPU path"
+                               % self.device)
+        ops.get_lib()                       # fail now, loudly, if the kernels are missing
+        self.page_size = int(page_size)
+        self.max_requests = int(max_requests)
+        if num_pages is None:
+            num_pages = (int(max_tokens) + self.page_size - 1) // self.page_size
+        self.num_pages = int(num_pages)
+
+        # ---- cache groups from the mixers' needs -------------------------------------
+        needs = model.cache_needs()
+        keyed: Dict[tuple, List[int]] = {}
+        for slot, need in enumerate(needs):
+            if need.kind == "kv":
+                keyed.setdefault((need.n_kv_heads, need.head_dim, need.window), []).append(slot)
+        self.groups: List[GroupSpec] = [
+            GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots))
+            for (nkv, dh, w), slots in keyed.items()]
+        if not self.groups:                  # a model without paged mixers still has a (tiny) page pool
+            self.groups = []
+        self.cache = CacheManager(self.groups, [self.num_pages] * len(self.groups), self.page_size,
+                                  self.max_requests, model.spec.max_positions)
+        self.storage = CacheStorage(self.groups, [self.num_pages] * len(self.groups), self.page_size,
+                                    self.runtime.dtype, self.device)
+        for slot, need in enumerate(needs):
+            if need.kind == "state":
+                self.storage.add_state(slot, self.max_requests, need.state_shape, need.state_dtype)
+        self._slot_group = {s: g for g, spec in enumerate(self.groups) for s in spec.slots}
+
+        self.ws = Workspace(self.device)
+        self._ring = _PinnedRing()
+        self._meta_dev: Optional[torch.Tensor] = None
+        self._tile_rows = ops.attention_prefill_tile_rows()
+        self.cu_count = torch.cuda.get_device_properties(self.device).multi_processor_count
+        self.steps_run = 0
+
+    # ---- construction -----------------------------------------------------------------
+    @classmethod
+    def from_dir(cls, model_dir: str, dtype=torch.bfloat16, device="cuda:0", max_tokens: Optional[int] = None,
+                 attention_impl: str = "auto", gemm_impl: str = "auto", max_context: Optional[int] = None,
+                 **kw):
+        cfg = config_from_dir(model_dir, max_tokens=max_context) if max_context else config_from_dir(model_dir)
+        rt = Runtime(dtype=dtype, device=device, attention_impl=attention_impl, gemm_impl=gemm_impl)
+        model = build_model(cfg.model_spec(), rt)
+        model.load_from_dir(model_dir)
+        if max_tokens is None:
+            max_tokens = model.spec.max_positions
+        eng = cls(model, max_tokens=max_tokens, **kw)
+        eng.config = cfg
+        return eng
+
+    # ---- requests -------------------------------------------------------------------------
+    def has_request(self, req_id) -> bool:
+        return self.cache.has_request(req_id)
+
+    def add_request(self, req_id) -> None:
+        slot = self.cache.admit(req_id)
+        self.storage.zero_state(slot)
+
+    def free(self, req_id) -> None:
+        if self.cache.has_request(req_id):
+            self.cache.release(req_id)
+
+    def length(self, req_id) -> int:
+        return self.cache.length(req_id)
+
+    # ---- the step ----------------------------------------------------------------------------
+    def step(self, entries: Sequence[StepEntry]):
+        """Run the entries' tokens as one batch.  Returns float32 logits
+        [number of wanted places, vocab] on the device, in the order of the entries and
+        of each entry's ``want`` (None when nothing is wanted).  The tensor is a
+        workspace view: it is valid until the next step."""
+        if not entries:
+            return None
+        vocab = self.model.spec.vocab_size
+        seen = set()
+        for e in entries:
+            if e.req_id in seen:
+                raise ValueError("request %r appears twice in one step" % (e.req_id,))
+            seen.add(e.req_id)
+            if len(e.tokens) == 0:
+                raise ValueError("request %r brings no tokens" % (e.req_id,))
+            for t in e.tokens:
+                if not (0 <= int(t) < vocab):
+                    raise ValueError("token id %r of request %r is outside the vocabulary (%d)" % (t, e.req_id, vocab))
+            for w in e.want:
+                if not (0 <= int(w) < len(e.tokens)):
+                    raise ValueError("wanted place %r of request %r is outside its %d tokens" % (w, e.req_id, len(e.tokens)))
+
+        # ---- room in the cache: all or nothing ------------------------------------------------
+        new_ids = [e.req_id for e in entries if not self.cache.has_request(e.req_id)]
+        if len(new_ids) > self.cache.slots.n_free:
+            raise OutOfPages("%d new requests but %d free state slots" % (len(new_ids), self.cache.slots.n_free))
+        need = [0] * len(self.groups)
+        for e in entries:
+            if self.cache.has_request(e.req_id):
+                per = self.cache.pages_needed(e.req_id, len(e.tokens))
+            else:
+                per = [(len(e.tokens) + self.page_size - 1) // self.page_size] * len(self.groups)
+            need = [a + b for a, b in zip(need, per)]
+        for g, n in enumerate(need):
+            if n > self.cache.free_pages(g):
+                raise OutOfPages("step needs %d pages of group %d, %d free" % (n, g, self.cache.free_pages(g)))
+        for rid in new_ids:
+            self.add_request(rid)
+        starts = [self.cache.append(e.req_id, len(e.tokens)) for e in entries]
+
+        ctx = self._build_context(entries, starts)
+        logits = self.model.forward(ctx)
+        for e in entries:
+            self.cache.trim(e.req_id)
+        self.steps_run += 1
+        return logits
+
+    # ---- packing the batch ------------------------------------------------------------------------
+    def _build_context(self, entries, starts) -> StepContext:
+        ps = self.page_size
+        R = len(entries)
+        T = sum(len(e.tokens) for e in entries)
+        tokens, positions, token_req, want_rows = [], [], [], []
+        decode_rows, tiles = [], []
+        req_start = [0]
+        max_ctx = 0
+        for r, (e, p0) in enumerate(zip(entries, starts)):
+            n = len(e.tokens)
+            row0 = req_start[-1]
+            tokens.extend(int(t) for t in e.tokens)
+            positions.extend(range(p0, p0 + n))
+            token_req.extend([r] * n)
+            want_rows.extend(row0 + int(w) for w in e.want)
+            if n == 1:
+                decode_rows.append(row0)
+                max_ctx = max(max_ctx, p0 + 1)
+            else:
+                for o in range(0, n, self._tile_rows):
+                    tiles.extend((r, row0 + o, min(self._tile_rows, n - o), p0 + o))
+            req_start.append(row0 + n)
+        state_slots = [self.cache.state_slot(e.req_id) for e in entries]
+
+        group_slots, group_tables, group_maxb = [], [], []
+        for g in range(len(self.groups)):
+            sl = []
+            maxb = 1
+            for e, p0 in zip(entries, starts):
+                table = self.cache.block_table(e.req_id, g)
+                maxb = max(maxb, len(table))
+                for p in range(p0, p0 + len(e.tokens)):
+                    sl.append(table[p // ps] * ps + p % ps)
+            bt = []
+            for e in entries:
+                table = self.cache.block_table(e.req_id, g)
+                bt.extend(max(p, 0) for p in table)      # pages given back are never read; keep the index valid
+                bt.extend([0] * (maxb - len(table)))
+            group_slots.append(sl)
+            group_tables.append(bt)
+            group_maxb.append(maxb)
+
+        sections = [("tokens", tokens), ("positions", positions), ("token_req", token_req),
+                    ("state_slots", state_slots), ("want_rows", want_rows), ("decode_rows", decode_rows),
+                    ("tiles", tiles)]
+        for g in range(len(self.groups)):
+            sections.append(("slots%d" % g, group_slots[g]))
+            sections.append(("tables%d" % g, group_tables[g]))
+        offsets, total = {}, 0
+        for name, data in sections:
+            offsets[name] = (total, len(data))
+            total += _align4(len(data))
+        host = self._ring.get(total)
+        flat: List[int] = []
+        for name, data in sections:
+            flat.extend(data)
+            flat.extend([0] * (_align4(len(data)) - len(data)))
+        host[:total] = torch.tensor(flat, dtype=torch.int32)
+        if self._meta_dev is None or self._meta_dev.numel() < total:
+            self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
+        dev = self._meta_dev
+        dev[:total].copy_(host[:total], non_blocking=True)
+        self._ring.mark()
+
+        def view(name):
+            o, n = offsets[name]
+            return dev[o:o + n]
+
+        ctx = StepContext()
+        ctx.T, ctx.R, ctx.page_size, ctx.ws = T, R, ps, self.ws
+        ctx.tokens, ctx.positions, ctx.token_req = view("tokens"), view("positions"), view("token_req")
+        ctx.state_slots = view("state_slots")
+        ctx.want_rows, ctx.n_want = view("want_rows"), len(want_rows)
+        ctx.decode_rows, ctx.n_decode_rows = view("decode_rows"), len(decode_rows)
+        ctx.decode_rows_identity = (len(decode_rows) == T)
+        ctx.prefill_tiles = view("tiles").view(-1, 4)
+        ctx.n_prefill_tiles = len(tiles) // 4
+        ctx.req_start, ctx.req_pos = req_start, list(starts)
+        ctx.req_len = [len(e.tokens) for e in entries]
+        ctx.req_ids = [e.req_id for e in entries]
+        ctx.host_state_slots = state_slots
+        ctx.max_position = max(positions)
+        ctx.max_context = max_ctx
+        ctx.cu_count = self.cu_count
+        for slot in range(self.model.spec.num_cache_slots()):
+            if slot in self._slot_group:
+                g = self._slot_group[slot]
+                k, v = self.storage.kv(slot)
+                ctx._views[slot] = LayerCacheView(k=k, v=v, slots=view("slots%d" % g),
+                                                  block_tables=view("tables%d" % g).view(R, group_maxb[g]))
+            else:
+                ctx._views[slot] = LayerCacheView(state=self.storage.state.get(slot))
+        return ctx
+
+    # ---- sampling --------------------------------------------------------------------------------------
+    def sample(self, logits, temperature=None, top_k=None, top_p=None, uniform=None) -> List[int]:
+        """Tokens for the rows of ``logits``.  With ``temperature`` None every row is
+        argmax; otherwise per-row lists of temperature, top_k, top_p and a uniform draw."""
+        R = logits.shape[0]
+        out = self.ws.buffer("sampled", (R,), torch.int32)
+        if temperature is None:
+            ops.sample(logits, out)
+        else:
+            f = torch.tensor([list(temperature), list(top_p), list(uniform)], dtype=torch.float32).to(self.device)
+            k = torch.tensor(list(top_k), dtype=torch.int32).to(self.device)
+            ops.sample(logits, out, f[0].contiguous(), k, f[1].contiguous(), f[2].contiguous())
+        return out.cpu().tolist()

@@ -1,0 +1,247 @@
+"""Python face of the HIP kernels: one function per kernel.  Each checks on the
+host that shapes, dtypes and strides are what the kernel and its grid assume,
+then launches on torch's current stream.  Nothing here computes on the CPU.
+"""
+import torch
+
+from .lib import KernelError, check, get_lib
+
+F32, BF16 = 0, 1
+_DT = {torch.float32: F32, torch.bfloat16: BF16}
+
+
+def dtype_code(dt) -> int:
+    try:
+        return _DT[dt]
+    except KeyError:
+        raise KernelError("dtype %s is not supported by the kernels (float32, bfloat16)" % dt)
+
+
+def _stream():
+    return torch.cuda.current_stream().cuda_stream
+
+
+def _need(cond, what):
+    if not cond:
+        raise KernelError(what)
+
+
+def _dev(*ts):
+    for t in ts:
+        if t is not None and not t.is_cuda:
+            raise KernelError("kernel operands must be on the GPU (got a %s tensor)" % t.device)
+
+
+def _i32(t, name):
+    _need(t.dtype == torch.int32 and t.is_contiguous(), "%s must be a contiguous int32 tensor" % name)
+
+
+def embed(tokens, table, out, scale: float):
+    """out[t, :] = table[tokens[t], :] * scale; out is float32 [T, d]."""
+    _dev(tokens, table, out)
+    _i32(tokens, "tokens")
+    T, d = out.shape
+    _need(tokens.numel() == T and table.dim() == 2 and table.shape[1] == d, "embed: shape mismatch")
+    _need(out.dtype == torch.float32 and out.is_contiguous() and table.is_contiguous(), "embed: layout")
+    check(get_lib().ic_embed(tokens.data_ptr(), table.data_ptr(), dtype_code(table.dtype), out.data_ptr(),
+                             T, d, float(scale), _stream()), "embed")
+    return out
+
+
+def rmsnorm(x, weight, out, eps: float, out_scale: float = 1.0, rows=None):
+    """out[r] = x[rows[r] or r] * rsqrt(mean(x^2) + eps) * weight * out_scale.  x is float32."""
+    _dev(x, weight, out, rows)
+    d = x.shape[-1]
+    n = out.shape[0]
+    _need(x.dtype == torch.float32 and x.is_contiguous() and out.is_contiguous(), "rmsnorm: layout")
+    _need(weight.dtype == torch.float32 and weight.numel() == d and out.shape[-1] == d, "rmsnorm: shape mismatch")
+    if rows is not None:
+        _i32(rows, "rows")
+        _need(rows.numel() == n, "rmsnorm: rows/out mismatch")
+    else:
+        _need(x.shape[0] == n, "rmsnorm: x/out mismatch")
+    check(get_lib().ic_rmsnorm(x.data_ptr(), rows.data_ptr() if rows is not None else None, weight.data_ptr(),
+                               out.data_ptr(), dtype_code(out.dtype), n, d, float(eps), float(out_scale),
+                               _stream()), "rmsnorm")
+    return out
+
+
+def add_rmsnorm(x, y, alpha: float, weight, out, eps: float):
+    """x += alpha * y (x float32, in place); out = rmsnorm(x) * weight."""
+    _dev(x, y, weight, out)
+    T, d = x.shape
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and out.is_contiguous(),
+          "add_rmsnorm: layout")
+    _need(tuple(y.shape) == (T, d) and tuple(out.shape) == (T, d) and weight.numel() == d
+          and weight.dtype == torch.float32, "add_rmsnorm: shape mismatch")
+    check(get_lib().ic_add_rmsnorm(x.data_ptr(), y.data_ptr(), dtype_code(y.dtype), float(alpha),
+                                   weight.data_ptr(), out.data_ptr(), dtype_code(out.dtype), T, d,
+                                   float(eps), _stream()), "add_rmsnorm")
+    return out
+
+
+def residual_add(x, y, alpha: float):
+    """x += alpha * y; x float32."""
+    _dev(x, y)
+    _need(x.dtype == torch.float32 and x.is_contiguous() and y.is_contiguous() and x.shape == y.shape,
+          "residual_add: layout")
+    check(get_lib().ic_residual_add(x.data_ptr(), y.data_ptr(), dtype_code(y.dtype), float(alpha),
+                                    x.numel(), _stream()), "residual_add")
+    return x
+
+
+def swiglu(gate_up, out):
+    """out[t, j] = up * silu(gate), gate = gate_up[t, j], up = gate_up[t, di + j]."""
+    _dev(gate_up, out)
+    T, di = out.shape
+    _need(tuple(gate_up.shape) == (T, 2 * di) and gate_up.is_contiguous() and out.is_contiguous()
+          and gate_up.dtype == out.dtype, "swiglu: layout")
+    check(get_lib().ic_swiglu(gate_up.data_ptr(), out.data_ptr(), dtype_code(out.dtype), T, di, _stream()),
+          "swiglu")
+    return out
+
+
+def rope_kv_write(qkv, positions, cos, sin, kcache, vcache, slots, n_heads, n_kv_heads, head_dim,
+                  rot_dim, page_size):
+    """Rotate the q heads of qkv[T, H] in place; rotate the k heads and copy the
+    v heads into cache slot ``slots[t]``.  n_kv_heads == 0: q only, no cache write."""
+    _dev(qkv, positions, cos, sin, kcache, vcache, slots)
+    T = qkv.shape[0]
+    _i32(positions, "positions")
+    _need(qkv.dim() == 2 and qkv.stride(1) == 1, "rope: qkv must be [T, H] with unit inner stride")
+    _need(qkv.shape[1] >= (n_heads + 2 * n_kv_heads) * head_dim, "rope: qkv row too short")
+    _need(positions.numel() == T, "rope: positions/qkv mismatch")
+    half = rot_dim // 2
+    if rot_dim > 0:
+        _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous()
+              and sin.is_contiguous() and cos.shape[-1] == half and sin.shape == cos.shape,
+              "rope: cos/sin must be float32 [max_pos, rot/2]")
+    if n_kv_heads > 0:
+        _i32(slots, "slots")
+        _need(slots.numel() == T, "rope: slots/qkv mismatch")
+        _need(kcache.dtype == qkv.dtype and vcache.dtype == qkv.dtype, "rope: cache dtype differs from qkv")
+        _need(kcache.is_contiguous() and vcache.is_contiguous()
+              and tuple(kcache.shape[1:]) == (n_kv_heads, page_size, head_dim)
+              and kcache.shape == vcache.shape, "rope: cache must be [pages, kv_heads, page_size, head_dim]")
+    check(get_lib().ic_rope_kv_write(
+        qkv.data_ptr(), dtype_code(qkv.dtype), positions.data_ptr(),
+        cos.data_ptr() if rot_dim > 0 else None, sin.data_ptr() if rot_dim > 0 else None,
+        kcache.data_ptr() if n_kv_heads > 0 else None, vcache.data_ptr() if n_kv_heads > 0 else None,
+        slots.data_ptr() if n_kv_heads > 0 else None,
+        T, qkv.stride(0), n_heads, n_kv_heads, head_dim, rot_dim, page_size, _stream()), "rope_kv_write")
+
+
+def _attn_common(q, out, kcache, vcache, block_tables, n_heads, n_kv_heads, head_dim, page_size):
+    _dev(q, out, kcache, vcache, block_tables)
+    _need(q.dim() == 2 and q.stride(1) == 1 and q.shape[1] >= n_heads * head_dim, "attention: q layout")
+    _need(out.dim() == 2 and out.stride(1) == 1 and out.shape[1] >= n_heads * head_dim, "attention: out layout")
+    _need(q.dtype == out.dtype == kcache.dtype == vcache.dtype, "attention: dtypes differ")
+    _need(kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape == vcache.shape
+          and tuple(kcache.shape[1:]) == (n_kv_heads, page_size, head_dim),
+          "attention: cache must be [pages, kv_heads, page_size, head_dim]")
+    _need(block_tables.dtype == torch.int32 and block_tables.dim() == 2 and block_tables.stride(1) == 1,
+          "attention: block_tables must be int32 [R, max_blocks]")
+    _need(n_heads % n_kv_heads == 0, "attention: heads not a multiple of kv heads")
+
+
+def attention_generic(q, out, kcache, vcache, block_tables, token_req, positions, n_heads, n_kv_heads,
+                      head_dim, page_size, scale: float, window: int = 0):
+    """out[t, h] = softmax over keys <= positions[t] (within the window) of q[t, h] . K, times V."""
+    _attn_common(q, out, kcache, vcache, block_tables, n_heads, n_kv_heads, head_dim, page_size)
+    _i32(token_req, "token_req")
+    _i32(positions, "positions")
+    T = q.shape[0]
+    _need(token_req.numel() == T and positions.numel() == T and out.shape[0] == T, "attention: T mismatch")
+    _need(head_dim <= 512, "attention: head size above 512")
+    check(get_lib().ic_attn_generic(
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype), kcache.data_ptr(),
+        vcache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), token_req.data_ptr(),
+        positions.data_ptr(), T, n_heads, n_kv_heads, head_dim, page_size, float(scale), int(window or 0),
+        _stream()), "attention_generic")
+
+
+def attention_decode_supported(dtype, head_dim: int) -> bool:
+    return bool(get_lib().ic_attn_decode_supported(dtype_code(dtype), head_dim))
+
+
+def attention_decode(q, out, kcache, vcache, block_tables, tok_list, n_tok, token_req, positions, part_acc,
+                     part_ml, n_heads, n_kv_heads, head_dim, page_size, scale: float, window: int, n_split: int):
+    """Split-key attention of the single tokens listed in tok_list (None: rows 0..n_tok-1)."""
+    _attn_common(q, out, kcache, vcache, block_tables, n_heads, n_kv_heads, head_dim, page_size)
+    _i32(token_req, "token_req")
+    _i32(positions, "positions")
+    if tok_list is not None:
+        _i32(tok_list, "tok_list")
+        _need(tok_list.numel() >= n_tok, "attention_decode: tok_list too short")
+    else:
+        _need(q.shape[0] >= n_tok, "attention_decode: fewer rows than tokens")
+    _need(part_acc.dtype == torch.float32 and part_acc.is_contiguous()
+          and part_acc.numel() >= n_tok * n_heads * n_split * head_dim, "attention_decode: part_acc too small")
+    _need(part_ml.dtype == torch.float32 and part_ml.is_contiguous()
+          and part_ml.numel() >= n_tok * n_heads * n_split * 2, "attention_decode: part_ml too small")
+    check(get_lib().ic_attn_decode(
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype), kcache.data_ptr(),
+        vcache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0),
+        tok_list.data_ptr() if tok_list is not None else None, token_req.data_ptr(), positions.data_ptr(),
+        part_acc.data_ptr(), part_ml.data_ptr(), n_tok, n_heads, n_kv_heads, head_dim, page_size,
+        float(scale), int(window or 0), int(n_split), _stream()), "attention_decode")
+
+
+def attention_prefill_supported(dtype, head_dim: int) -> bool:
+    return bool(get_lib().ic_attn_prefill_supported(dtype_code(dtype), head_dim))
+
+
+def attention_prefill_tile_rows() -> int:
+    return get_lib().ic_attn_prefill_tile_rows()
+
+
+def attention_prefill(q, out, kcache, vcache, block_tables, tiles, n_tiles, n_heads, n_kv_heads, head_dim,
+                      page_size, scale: float, window: int = 0):
+    """Matrix-core attention of prompt portions.  tiles: int32 [n, 4] rows of
+    (request row in block_tables, first token row, rows <= tile_rows, first position)."""
+    _attn_common(q, out, kcache, vcache, block_tables, n_heads, n_kv_heads, head_dim, page_size)
+    _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.dim() == 2 and tiles.shape[1] == 4
+          and tiles.shape[0] >= n_tiles, "attention_prefill: tiles must be int32 [n, 4]")
+    check(get_lib().ic_attn_prefill(
+        q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype), kcache.data_ptr(),
+        vcache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), tiles.data_ptr(), n_tiles,
+        n_heads, n_kv_heads, head_dim, page_size, float(scale), int(window or 0), _stream()),
+        "attention_prefill")
+
+
+def sample(logits, out, temperature=None, top_k=None, top_p=None, uniform=None):
+    """out[r] = token sampled from logits[r] (float32 [R, V]).  temperature None: argmax."""
+    _dev(logits, out, temperature, top_k, top_p, uniform)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "sample: logits must be float32 rows")
+    _i32(out, "out")
+    _need(out.numel() >= R, "sample: out too short")
+    if temperature is not None:
+        _need(temperature.dtype == torch.float32 and top_p.dtype == torch.float32
+              and uniform.dtype == torch.float32 and top_k.dtype == torch.int32, "sample: parameter dtypes")
+        _need(min(temperature.numel(), top_k.numel(), top_p.numel(), uniform.numel()) >= R,
+              "sample: parameter arrays too short")
+    p = lambda t: t.data_ptr() if t is not None else None
+    check(get_lib().ic_sample(logits.data_ptr(), logits.stride(0), R, V, p(temperature), p(top_k), p(top_p),
+                              p(uniform), out.data_ptr(), _stream()), "sample")
+    return out
+
+
+def gemm_nt_supported(a_dtype, w_dtype, c_dtype) -> bool:
+    try:
+        return bool(get_lib().ic_gemm_nt_supported(dtype_code(a_dtype), dtype_code(w_dtype), dtype_code(c_dtype)))
+    except KernelError:
+        return False
+
+
+def gemm_nt(a, w, out, alpha: float = 1.0):
+    """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation)."""
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K and tuple(out.shape) == (M, N), "gemm_nt: shape mismatch")
+    _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm_nt: inner strides must be 1")
+    check(get_lib().ic_gemm_nt(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
+                               out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),
+                               out.stride(0), float(alpha), _stream()), "gemm_nt")
+    return out

@@ -1,0 +1,108 @@
+"""Softmax attention over the paged cache (MHA or grouped-query).
+
+Per layer the reference does (src/models/jiuge/jiuge.cpp:200-236): fused QKV
+projection, rotary on q and k heads, append k and v to the cache, scores
+(1/sqrt(dh)) Q K^T over keys 0..t-1, causal softmax aligned to the bottom right,
+P V, output projection.  Query head h uses key/value head h // (nh/nkvh)
+(jiuge.cpp:210-213).  Here the scores never reach memory: one of three kernels
+walks the cache with a float32 running softmax,
+  * a split-key kernel for rows that are a request's single new token,
+  * a matrix-core kernel for prompt portions (bfloat16, head size 64 or 128),
+  * the general kernel for everything else and for float32 portions.
+"""
+import torch
+
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import CacheNeed, Mixer, build_part, register_part
+from .linear import linear
+
+
+@register_part("mixer", "attention")
+class Attention(Mixer):
+    def __init__(self, name, runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
+                 softmax_scale: float, position_encoding, window=None, shared_kv: bool = False):
+        super().__init__(name, runtime)
+        if num_heads % num_kv_heads:
+            raise ValueError("attention: %d heads are not a multiple of %d kv heads" % (num_heads, num_kv_heads))
+        if head_dim % 16:
+            raise ValueError("attention: head size %d is not a multiple of 16" % head_dim)
+        if head_dim > 512:
+            raise ValueError("attention: head size %d above 512" % head_dim)
+        self.hidden_size = hidden_size
+        self.nh, self.nkvh, self.dh = num_heads, num_kv_heads, head_dim
+        self.scale = float(softmax_scale)
+        self.window = int(window) if window else 0
+        self.shared_kv = bool(shared_kv)          # reads another entry's cache: projects q only
+        self.pos_enc = position_encoding if not hasattr(position_encoding, "kind") \
+            else build_part("position_encoding", position_encoding, runtime)
+        self.w_qkv = None
+        self.w_o = None
+
+    def sub_parts(self):
+        return (self.pos_enc,)
+
+    def cache_need(self):
+        return CacheNeed("kv", self.nkvh, self.dh, self.window or None)
+
+    # ---- weights: names of scripts/jiuge.py:45-63 ------------------------------
+    def weight_specs(self):
+        n = self.name
+        specs = {
+            n + "q_proj.weight": WeightSpec((self.nh * self.dh, self.hidden_size)),
+            n + "o_proj.weight": WeightSpec((self.hidden_size, self.nh * self.dh)),
+        }
+        if not self.shared_kv:
+            specs[n + "k_proj.weight"] = WeightSpec((self.nkvh * self.dh, self.hidden_size))
+            specs[n + "v_proj.weight"] = WeightSpec((self.nkvh * self.dh, self.hidden_size))
+        return specs
+
+    def load_weights(self, tensors):
+        n = self.name
+        names = ["q_proj.weight"] + ([] if self.shared_kv else ["k_proj.weight", "v_proj.weight"])
+        mats = [tensors[n + s] for s in names]
+        if len({m.dtype for m in mats}) > 1:
+            mats = [m.to(torch.float32) for m in mats]
+        # rows [Q; K; V] of one fused projection (jiuge.py:237-239), unpermuted
+        self.w_qkv = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
+        self.w_o = tensors[n + "o_proj.weight"]
+
+    # ---- forward ---------------------------------------------------------------------
+    def forward(self, h, ctx, cache):
+        rt = self.runtime
+        T = h.shape[0]
+        nkv = 0 if (self.shared_kv or not cache.writes) else self.nkvh
+        width = (self.nh + 2 * (0 if self.shared_kv else self.nkvh)) * self.dh
+        qkv = ctx.ws.buffer("qkv", (T, width), rt.dtype)
+        linear(h, self.w_qkv, qkv, rt.gemm_impl)
+        self.pos_enc.rotate_and_store(qkv, ctx, cache, self.nh, nkv, self.dh)
+        out = ctx.ws.buffer("attn_out", (T, self.nh * self.dh), rt.dtype)
+        self._attend(qkv, out, ctx, cache)
+        y = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
+        linear(out, self.w_o, y, rt.gemm_impl)
+        return y
+
+    def _attend(self, q, out, ctx, cache):
+        rt = self.runtime
+        args = (self.nh, self.nkvh, self.dh, ctx.page_size)
+        fast = rt.attention_impl == "auto"
+        dec_ok = fast and ops.attention_decode_supported(rt.dtype, self.dh)
+        pre_ok = fast and ops.attention_prefill_supported(rt.dtype, self.dh)
+        n_dec, n_tiles = ctx.n_decode_rows, ctx.n_prefill_tiles
+        use_dec = dec_ok and n_dec > 0 and (pre_ok or n_tiles == 0)
+        use_pre = pre_ok and n_tiles > 0 and (dec_ok or n_dec == 0)
+        if not ((use_dec or n_dec == 0) and (use_pre or n_tiles == 0)):
+            ops.attention_generic(q, out, cache.k, cache.v, cache.block_tables, ctx.token_req, ctx.positions,
+                                  *args, self.scale, self.window)
+            return
+        if use_dec:
+            n_split = ctx.decode_splits(self.nkvh, self.window)
+            part_acc = ctx.ws.buffer("attn_part_acc", (n_dec * self.nh * n_split * self.dh,), torch.float32)
+            part_ml = ctx.ws.buffer("attn_part_ml", (n_dec * self.nh * n_split * 2,), torch.float32)
+            ops.attention_decode(q, out, cache.k, cache.v, cache.block_tables,
+                                 None if ctx.decode_rows_identity else ctx.decode_rows, n_dec,
+                                 ctx.token_req, ctx.positions, part_acc, part_ml, *args, self.scale,
+                                 self.window, n_split)
+        if use_pre:
+            ops.attention_prefill(q, out, cache.k, cache.v, cache.block_tables, ctx.prefill_tiles, n_tiles,
+                                  *args, self.scale, self.window)

@@ -1,0 +1,152 @@
+"""Interfaces of the parts a layer is put together from, and their registry.
+
+Categories: ``mixer`` (attention here), ``feed_forward``, ``norm``,
+``position_encoding``, ``block`` (the arrangement of the others in a layer),
+``embedding`` and ``head``.  A part is built from a ``PartSpec``: its class is
+looked up by ``(category, kind)`` and called as ``cls(name, runtime, **params)``.
+A part sees its own parameters, the step's batch description and the cache
+view it is handed; it never sees the model or its configuration.
+"""
+from dataclasses import dataclass
+from typing import Callable, Dict, Optional, Tuple
+
+import torch
+
+from ..config.spec import PartSpec
+from ..weights.loader import WeightSpec
+
+CATEGORIES = ("mixer", "feed_forward", "norm", "position_encoding", "block", "embedding", "head")
+_REGISTRY: Dict[str, Dict[str, type]] = {c: {} for c in CATEGORIES}
+
+
+@dataclass(frozen=True)
+class Runtime:
+    """What every part needs to know about where and how it computes."""
+    dtype: torch.dtype                 # compute dtype of activations and cache: bfloat16 or float32
+    device: object                     # torch device of weights and buffers
+    attention_impl: str = "auto"       # "auto": tiled kernels where they apply; "generic": the general kernel only
+    gemm_impl: str = "auto"            # "auto": own kernel for few rows; "library": always the library GEMM
+
+
+@dataclass(frozen=True)
+class CacheNeed:
+    """What a mixer needs from the cache manager.
+    kind 'kv': paged keys and values of n_kv_heads x head_dim, all of them or a window;
+    kind 'state': a fixed-size tensor of ``state_shape`` per request;
+    kind 'none': nothing."""
+    kind: str = "none"
+    n_kv_heads: int = 0
+    head_dim: int = 0
+    window: Optional[int] = None
+    state_shape: Tuple[int, ...] = ()
+    state_dtype: torch.dtype = torch.float32
+
+
+def register_part(category: str, kind: str) -> Callable:
+    if category not in _REGISTRY:
+        raise KeyError("unknown part category %r (have %s)" % (category, ", ".join(CATEGORIES)))
+
+    def _do(cls):
+        _REGISTRY[category][kind] = cls
+        return cls
+    return _do
+
+
+def registered_parts(category: str):
+    return sorted(_REGISTRY[category])
+
+
+def build_part(category: str, spec: PartSpec, runtime: Runtime, memo: Optional[dict] = None):
+    """Instantiate the part a spec names.  ``memo`` (id(spec) -> part) lets
+    several layers share one instance of the same spec object."""
+    if memo is not None and id(spec) in memo:
+        return memo[id(spec)]
+    try:
+        cls = _REGISTRY[category][spec.kind]
+    except KeyError:
+        raise KeyError("no %s part of kind %r; registered: %s"
+                       % (category, spec.kind, ", ".join(registered_parts(category))))
+    part = cls(spec.name, runtime, **spec.params)
+    if memo is not None:
+        memo[id(spec)] = part
+    return part
+
+
+class Part:
+    """Base of all parts."""
+    category = ""
+
+    def __init__(self, name: str, runtime: Runtime):
+        self.name = name
+        self.runtime = runtime
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        """Full tensor name -> what is expected of it."""
+        return {}
+
+    def load_weights(self, tensors: Dict[str, torch.Tensor]) -> None:
+        """Take this part's tensors (keys as in weight_specs) from ``tensors``."""
+
+    def sub_parts(self):
+        return ()
+
+
+class Norm(Part):
+    category = "norm"
+
+    def forward(self, x, out, rows=None, out_scale: float = 1.0):
+        """out[r] = norm(x[rows[r] or r]) * out_scale; x is the float32 residual stream."""
+        raise NotImplementedError
+
+    def forward_add(self, x, y, alpha: float, out):
+        """x += alpha * y, then out = norm(x).  Parts without a fused kernel inherit this."""
+        from ..kernels import ops
+        ops.residual_add(x, y, alpha)
+        return self.forward(x, out)
+
+
+class PositionEncoding(Part):
+    category = "position_encoding"
+
+    def rotate_and_store(self, qkv, ctx, cache, n_heads: int, n_kv_heads: int, head_dim: int):
+        """Encode positions into the q (and k) heads of qkv[T, H] in place and,
+        when n_kv_heads > 0, write k and v into ``cache`` at the step's slots."""
+        raise NotImplementedError
+
+
+class Mixer(Part):
+    category = "mixer"
+
+    def cache_need(self) -> CacheNeed:
+        return CacheNeed()
+
+    def forward(self, h, ctx, cache):
+        """h: [T, hidden] normed input in the compute dtype; returns [T, hidden]."""
+        raise NotImplementedError
+
+
+class FeedForward(Part):
+    category = "feed_forward"
+
+    def forward(self, h, ctx):
+        raise NotImplementedError
+
+
+class Block(Part):
+    """Arrangement of a mixer and a feed-forward around the residual stream.
+    ``pending`` is a branch output whose residual add is still owed, as
+    ``(y, alpha)``; a block may hand its last add on to the next block's norm."""
+    category = "block"
+
+    def __init__(self, name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm):
+        super().__init__(name, runtime)
+        self.mixer = mixer
+        self.mixer_norm = mixer_norm
+        self.feed_forward = feed_forward
+        self.feed_forward_norm = feed_forward_norm
+
+    def sub_parts(self):
+        return (self.mixer, self.mixer_norm, self.feed_forward, self.feed_forward_norm)
+
+    def forward(self, x, pending, ctx, cache):
+        raise NotImplementedError

@@ -1,0 +1,66 @@
+"""Token embedding and output head.
+
+Embedding: x = E[token] * scale_emb (scripts/jiuge.py:193-197; gather at
+src/models/jiuge/jiuge.cpp:164-168).  The scale is applied at gather time, so a
+tied table is held once.  Head: logits = (norm(x) * logit_scale) W^T in
+float32 out (jiuge.py:198-207, jiuge.cpp:262-264,270-278), only for the rows
+that are asked for.  Which tensor backs which table follows the reference: the
+embedding falls back to lm_head.weight and the head to model.embed_tokens.weight
+when its own tensor is absent (jiuge.py:182-191).
+"""
+import torch
+
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import Part, register_part
+from .linear import linear
+
+
+@register_part("embedding", "embedding")
+class Embedding(Part):
+    category = "embedding"
+
+    def __init__(self, name, runtime, vocab_size: int, hidden_size: int, scale: float = 1.0,
+                 fallback_name=None):
+        super().__init__(name, runtime)
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.scale = float(scale)
+        self.fallback = fallback_name + "weight" if fallback_name else None
+        self.table = None
+
+    def weight_specs(self):
+        return {self.name + "weight": WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback)}
+
+    def load_weights(self, tensors):
+        self.table = tensors[self.name + "weight"]
+
+    def forward(self, tokens, x):
+        return ops.embed(tokens, self.table, x, self.scale)
+
+
+@register_part("head", "lm_head")
+class LMHead(Part):
+    category = "head"
+
+    def __init__(self, name, runtime, vocab_size: int, hidden_size: int, logit_scale: float = 1.0,
+                 fallback_name=None):
+        super().__init__(name, runtime)
+        self.vocab_size, self.hidden_size = vocab_size, hidden_size
+        self.logit_scale = float(logit_scale)
+        self.fallback = fallback_name + "weight" if fallback_name else None
+        self.weight = None
+
+    def weight_specs(self):
+        return {self.name + "weight": WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback)}
+
+    def load_weights(self, tensors):
+        self.weight = tensors[self.name + "weight"]
+
+    def forward(self, x, rows, final_norm, ctx):
+        """Float32 logits [len(rows), vocab] of the residual rows ``rows``."""
+        n = rows.numel()
+        h = ctx.ws.buffer("head_in", (n, self.hidden_size), self.runtime.dtype)
+        final_norm.forward(x, h, rows=rows, out_scale=self.logit_scale)
+        logits = ctx.ws.buffer("logits", (n, self.vocab_size), torch.float32)
+        linear(h, self.weight, logits, self.runtime.gemm_impl)
+        return logits

@@ -1,0 +1,52 @@
+"""y = x W^T for weights stored [out, in] (the checkpoint's layout; the
+reference views them transposed, src/models/jiuge/jiuge_weight.hpp:51-54).
+
+The matrix product itself is a library routine for many rows, as in the
+reference (inference_context.cpp:59-79 calls the library's Gemm), and the
+package's own matrix-core kernel for few rows (decoding, the output head).
+float32 operands always go to the library with reduced-precision matrix modes
+switched off.
+"""
+import torch
+
+from ..kernels import ops
+
+# float32 products must be true float32.
+torch.backends.cuda.matmul.allow_tf32 = False
+torch.backends.cudnn.allow_tf32 = False
+
+FEW_ROWS = 64
+_mm_out_dtype_ok = None
+
+
+def _library_mm_f32_out(x, w, out):
+    """bfloat16 operands, float32 result: the library's mixed-output product when it has one."""
+    global _mm_out_dtype_ok
+    if _mm_out_dtype_ok is None:
+        try:
+            torch.mm(x[:1], w[:1].t(), out_dtype=torch.float32)
+            _mm_out_dtype_ok = True
+        except Exception:
+            _mm_out_dtype_ok = False
+    if _mm_out_dtype_ok:
+        out.copy_(torch.mm(x, w.t(), out_dtype=torch.float32))
+    else:
+        ops.gemm_nt(x, w, out)
+
+
+def linear(x, w, out, impl: str = "auto"):
+    """out[M, N] = x[M, K] @ w[N, K]^T.  out may be float32 when x is bfloat16."""
+    if w.dtype != x.dtype:
+        # a matrix stored in 32-bit stays so: compute this product in float32
+        tmp = torch.mm(x.to(torch.float32), w.to(torch.float32).t())
+        out.copy_(tmp)
+        return out
+    M = x.shape[0]
+    if x.dtype == torch.bfloat16:
+        if (impl == "auto" and M <= FEW_ROWS) and ops.gemm_nt_supported(x.dtype, w.dtype, out.dtype):
+            return ops.gemm_nt(x, w, out)
+        if out.dtype == torch.float32:
+            _library_mm_f32_out(x, w, out)
+            return out
+    torch.mm(x, w.t(), out=out)
+    return out

@@ -1,0 +1,125 @@
+"""The layered model: an embedding, layers run in the order a list gives, a
+final norm and a head.  Built from a ``ModelSpec``; knows no architecture.
+
+Forward of one step (src/models/jiuge/jiuge.cpp:164-168,195-258,261-278 is the
+reference's): gather embeddings into the float32 residual stream, run the
+schedule, settle the last residual add, then normalise and project only the
+rows whose logits are wanted.
+"""
+from typing import Dict, List
+
+import torch
+
+from ..config.spec import ModelSpec
+from ..kernels import ops
+from ..weights.loader import WeightSpec, load_weights
+from .base import CacheNeed, Runtime, build_part
+
+
+class DecoderModel:
+    def __init__(self, spec: ModelSpec, runtime: Runtime):
+        self.spec = spec
+        self.runtime = runtime
+        memo = {}
+        self.embedding = build_part("embedding", spec.embedding, runtime, memo)
+        self.layers = []
+        for ls in spec.layers:
+            mixer = build_part("mixer", ls.mixer, runtime, memo)
+            ffn = build_part("feed_forward", ls.feed_forward, runtime, memo)
+            n1 = build_part("norm", ls.mixer_norm, runtime, memo)
+            n2 = build_part("norm", ls.feed_forward_norm, runtime, memo)
+            from .base import _REGISTRY
+            try:
+                block_cls = _REGISTRY["block"][ls.block.kind]
+            except KeyError:
+                raise KeyError("no block part of kind %r" % ls.block.kind)
+            self.layers.append(block_cls(ls.block.name, runtime, mixer=mixer, mixer_norm=n1, feed_forward=ffn,
+                                         feed_forward_norm=n2, **ls.block.params))
+        self.final_norm = build_part("norm", spec.final_norm, runtime, memo)
+        self.head = build_part("head", spec.head, runtime, memo)
+        self.schedule = list(spec.schedule)
+        for e in self.schedule:
+            if not (0 <= e.layer < len(self.layers)):
+                raise ValueError("run order names layer %d, the model has %d" % (e.layer, len(self.layers)))
+        writers = {}
+        for e in self.schedule:
+            if e.writes_cache:
+                if e.cache in writers:
+                    raise ValueError("cache slot %d is written by two entries of the run order" % e.cache)
+                writers[e.cache] = e.layer
+        for e in self.schedule:
+            if not e.writes_cache and e.cache not in writers:
+                raise ValueError("cache slot %d is read but never written" % e.cache)
+        self._writers = writers
+
+    # ---- parts and weights ---------------------------------------------------------
+    def all_parts(self):
+        seen, out = set(), []
+
+        def walk(p):
+            if id(p) in seen:
+                return
+            seen.add(id(p))
+            out.append(p)
+            for s in p.sub_parts():
+                walk(s)
+        walk(self.embedding)
+        for l in self.layers:
+            walk(l)
+        walk(self.final_norm)
+        walk(self.head)
+        return out
+
+    def weight_specs(self) -> Dict[str, WeightSpec]:
+        specs: Dict[str, WeightSpec] = {}
+        for p in self.all_parts():
+            for name, s in p.weight_specs().items():
+                if name in specs and specs[name] != s:
+                    raise ValueError("tensor %s is wanted with two different specs" % name)
+                specs[name] = s
+        return specs
+
+    def load_weights(self, tensors: Dict[str, torch.Tensor]) -> None:
+        for p in self.all_parts():
+            p.load_weights(tensors)
+
+    def load_from_dir(self, model_dir: str) -> None:
+        tensors = load_weights(model_dir, self.weight_specs(), self.runtime.dtype, self.runtime.device)
+        self.load_weights(tensors)
+
+    # ---- cache needs ------------------------------------------------------------------
+    def cache_needs(self) -> List[CacheNeed]:
+        """One need per cache slot, in slot order."""
+        n = self.spec.num_cache_slots()
+        needs = [CacheNeed() for _ in range(n)]
+        for slot, layer in self._writers.items():
+            needs[slot] = self.layers[layer].mixer.cache_need()
+        return needs
+
+    def weight_bytes(self) -> int:
+        seen, total = set(), 0
+        for p in self.all_parts():
+            for v in vars(p).values():
+                if isinstance(v, torch.Tensor) and v.data_ptr() not in seen:
+                    seen.add(v.data_ptr())
+                    total += v.numel() * v.element_size()
+        return total
+
+    # ---- one step ------------------------------------------------------------------------
+    def forward(self, ctx):
+        """Runs ctx.T tokens; returns float32 logits [len(ctx.want_rows), vocab] or None."""
+        T = ctx.T
+        x = ctx.ws.buffer("residual", (T, self.spec.hidden_size), torch.float32)
+        self.embedding.forward(ctx.tokens, x)
+        pending = None
+        for e in self.schedule:
+            pending = self.layers[e.layer].forward(x, pending, ctx, ctx.cache_view(e))
+        if ctx.n_want == 0:
+            return None
+        if pending is not None:
+            ops.residual_add(x, pending[0], pending[1])
+        return self.head.forward(x, ctx.want_rows, self.final_norm, ctx)
+
+
+def build_model(spec: ModelSpec, runtime: Runtime) -> DecoderModel:
+    return DecoderModel(spec, runtime)

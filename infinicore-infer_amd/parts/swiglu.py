@@ -1,0 +1,50 @@
+"""Dense SwiGLU feed-forward: down( up(h) * silu(gate(h)) ).
+
+The reference fuses gate and up into one projection with rows [gate; up]
+(scripts/jiuge.py:311-323), applies swiglu(out=gate, up, gate)
+(src/models/jiuge/jiuge.cpp:247-248) and projects down (jiuge.cpp:249).  No
+biases.  The activation is computed in float32 inside the kernel.
+"""
+import torch
+
+from ..kernels import ops
+from ..weights.loader import WeightSpec
+from .base import FeedForward, register_part
+from .linear import linear
+
+
+@register_part("feed_forward", "swiglu")
+class SwiGLU(FeedForward):
+    def __init__(self, name, runtime, hidden_size: int, intermediate_size: int):
+        super().__init__(name, runtime)
+        self.hidden_size = hidden_size
+        self.intermediate_size = intermediate_size
+        self.w_gate_up = None
+        self.w_down = None
+
+    def weight_specs(self):
+        n, d, di = self.name, self.hidden_size, self.intermediate_size
+        return {
+            n + "gate_proj.weight": WeightSpec((di, d)),
+            n + "up_proj.weight": WeightSpec((di, d)),
+            n + "down_proj.weight": WeightSpec((d, di)),
+        }
+
+    def load_weights(self, tensors):
+        n = self.name
+        g, u = tensors[n + "gate_proj.weight"], tensors[n + "up_proj.weight"]
+        if g.dtype != u.dtype:
+            g, u = g.to(torch.float32), u.to(torch.float32)
+        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        self.w_down = tensors[n + "down_proj.weight"]
+
+    def forward(self, h, ctx):
+        rt = self.runtime
+        T = h.shape[0]
+        gate_up = ctx.ws.buffer("gate_up", (T, 2 * self.intermediate_size), rt.dtype)
+        linear(h, self.w_gate_up, gate_up, rt.gemm_impl)
+        act = ctx.ws.buffer("ffn_act", (T, self.intermediate_size), rt.dtype)
+        ops.swiglu(gate_up, act)
+        y = ctx.ws.buffer("ffn_out", (T, self.hidden_size), rt.dtype)
+        linear(act, self.w_down, y, rt.gemm_impl)
+        return y
