@@ -58,7 +58,8 @@ def test_replay_modes(tmp_path_factory, name, dname, dtype, tol, mode):
     ref = _reference(folder, name, requests, dtype == torch.bfloat16)
     got = H.run_trace(engine, steps)
     assert len(got) == sum(len(t) for t in requests.values())
-    H.compare(got, ref, tol, "%s %s %s" % (name, dname, mode))
+    worst = H.compare(got, ref, tol, "%s %s %s" % (name, dname, mode))
+    print("worst error %.3g at %s (allowed %.3g)" % (worst[0], worst[1], tol))
     engine.cache.check_invariants()
     assert not engine.cache.requests, "every request was ended"
     for g in range(len(engine.groups)):

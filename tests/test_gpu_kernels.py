@@ -1,0 +1,383 @@
+"""Each HIP kernel alone against a plain float64 reference of the same op, at
+sizes other than the tiny models': widths and vocabularies that are no power of
+two, head sizes in steps of 16, odd numbers of heads and groups."""
+import math
+
+import pytest
+import torch
+
+import plain_model as P
+
+pytestmark = pytest.mark.gpu
+
+DEV = "cuda:0"
+DT = [torch.float32, torch.bfloat16]
+
+
+def _ops():
+    from infinicore_infer_amd.kernels import ops
+    return ops
+
+
+def _tol(dtype):
+    return 2e-6 if dtype == torch.float32 else 1e-2
+
+
+def _close(got, want, dtype, scale=None, factor=1.0):
+    got, want = got.double().cpu(), want.double().cpu()
+    s = float(want.abs().max()) if scale is None else scale
+    err = float((got - want).abs().max()) / max(s, 1e-30)
+    assert math.isfinite(err) and err <= _tol(dtype) * factor, "error %.3g of the largest value" % err
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,d,V", [(1, 64, 50), (37, 200, 331), (300, 2304, 1000)])
+def test_embed(dtype, T, d, V):
+    g = torch.Generator().manual_seed(1)
+    table = torch.randn(V, d, generator=g).to(dtype)
+    tok = torch.randint(0, V, (T,), generator=g, dtype=torch.int32)
+    out = torch.empty(T, d, device=DEV)
+    _ops().embed(tok.to(DEV), table.to(DEV), out, 12.0)
+    want = P.plain_embedding(table, tok.tolist(), 12.0)
+    _close(out, want, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,d,eps", [(1, 64, 1e-5), (33, 200, 1e-6), (17, 2304, 1e-5), (5, 4097, 1e-2)])
+def test_rmsnorm(dtype, T, d, eps):
+    g = torch.Generator().manual_seed(2)
+    x = torch.randn(T, d, generator=g) * 3
+    x[0] *= 1e-3                      # a tiny row: eps inside the root matters there
+    w = 1 + 0.1 * torch.randn(d, generator=g)
+    out = torch.empty(T, d, dtype=dtype, device=DEV)
+    _ops().rmsnorm(x.to(DEV), w.to(DEV), out, eps)
+    _close(out, P.plain_rmsnorm(x, w, eps), dtype)
+    # library routine for the same formula
+    lib = torch.nn.functional.rms_norm(x.double(), (d,), w.double(), eps)
+    _close(out, lib, dtype)
+    # gathered rows with an output scale
+    rows = torch.tensor([T - 1, 0, T // 2], dtype=torch.int32)
+    out2 = torch.empty(3, d, dtype=dtype, device=DEV)
+    _ops().rmsnorm(x.to(DEV), w.to(DEV), out2, eps, 4.0, rows.to(DEV))
+    _close(out2, P.plain_rmsnorm(x[rows.long()], w, eps) * 4.0, dtype)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,d", [(3, 96), (40, 200), (9, 2304)])
+def test_add_rmsnorm_and_residual_add(dtype, T, d):
+    g = torch.Generator().manual_seed(3)
+    x = torch.randn(T, d, generator=g)
+    y = torch.randn(T, d, generator=g).to(dtype)
+    w = 1 + 0.1 * torch.randn(d, generator=g)
+    xd = x.to(DEV).clone()
+    out = torch.empty(T, d, dtype=dtype, device=DEV)
+    _ops().add_rmsnorm(xd, y.to(DEV), 0.7, w.to(DEV), out, 1e-5)
+    xs = x.double() + 0.7 * y.double()
+    _close(xd, xs, torch.float32)
+    _close(out, P.plain_rmsnorm(xs, w, 1e-5), dtype)
+    xd2 = x.to(DEV).clone()
+    _ops().residual_add(xd2, y.to(DEV), 0.7)
+    _close(xd2, xs, torch.float32)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("T,di", [(1, 160), (29, 344), (7, 5760)])
+def test_swiglu(dtype, T, di):
+    g = torch.Generator().manual_seed(4)
+    gu = (torch.randn(T, 2 * di, generator=g) * 2).to(dtype)
+    out = torch.empty(T, di, dtype=dtype, device=DEV)
+    _ops().swiglu(gu.to(DEV), out)
+    want = P.plain_swiglu(gu[:, :di], gu[:, di:])
+    _close(out, want, dtype)
+    lib = torch.nn.functional.silu(gu[:, :di].double()) * gu[:, di:].double()
+    _close(out, lib, dtype)
+    # swapped arguments must not pass
+    wrong = P.plain_swiglu(gu[:, di:], gu[:, :di])
+    assert float((out.double().cpu() - wrong).abs().max()) > 0.1
+
+
+# ---------------------------------------------------------------------------
+def _paged(k, v, page_size, dtype, seed=0, extra_pages=3):
+    """Scatter contiguous k, v [t, nkvh, dh] into shuffled pages; returns planes and the block table."""
+    t, nkvh, dh = k.shape
+    n_pages = (t + page_size - 1) // page_size
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_pages + extra_pages, generator=g)[:n_pages]
+    kc = torch.full((n_pages + extra_pages, nkvh, page_size, dh), float("nan")).to(dtype)
+    vc = torch.full_like(kc, float("nan"))
+    for j in range(t):
+        kc[perm[j // page_size], :, j % page_size] = k[j].to(dtype)
+        vc[perm[j // page_size], :, j % page_size] = v[j].to(dtype)
+    return kc, vc, perm.to(torch.int32)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("nh,nkvh,dh,rot,page", [(4, 2, 16, 16, 16), (3, 3, 32, 32, 32), (6, 2, 64, 64, 16),
+                                                  (5, 1, 48, 32, 16), (2, 2, 128, 128, 64)])
+def test_rope_kv_write(dtype, nh, nkvh, dh, rot, page):
+    g = torch.Generator().manual_seed(5)
+    T, max_pos = 23, 300
+    H = (nh + 2 * nkvh) * dh
+    qkv = torch.randn(T, H, generator=g).to(dtype)
+    pos = torch.randint(0, max_pos, (T,), generator=g, dtype=torch.int32)
+    n_pages = 6
+    slots = torch.randperm(n_pages * page, generator=g)[:T].to(torch.int32)
+    half = rot // 2
+    sin, cos = P.plain_rope_tables(rot, 10000.0, max_pos)
+    kc = torch.zeros(n_pages, nkvh, page, dh, dtype=dtype, device=DEV)
+    vc = torch.zeros_like(kc)
+    q_dev = qkv.to(DEV).clone()
+    _ops().rope_kv_write(q_dev, pos.to(DEV), cos.float().to(DEV), sin.float().to(DEV), kc, vc, slots.to(DEV),
+                         nh, nkvh, dh, rot, page)
+
+    def rot_half(x):          # pairs (j, j + rot/2) of each head; dims beyond rot pass through
+        x = x.double()
+        a, b = x[..., :half], x[..., half:rot]
+        c, s = cos[pos.long()][:, None, :], sin[pos.long()][:, None, :]
+        return torch.cat([a * c - b * s, a * s + b * c, x[..., rot:]], dim=-1)
+
+    heads = qkv.double().reshape(T, nh + 2 * nkvh, dh)
+    want_q = rot_half(heads[:, :nh])
+    want_k = rot_half(heads[:, nh:nh + nkvh])
+    want_v = heads[:, nh + nkvh:]
+    got = q_dev.cpu().double().reshape(T, nh + 2 * nkvh, dh)
+    _close(got[:, :nh], want_q, dtype)
+    kc_c, vc_c = kc.cpu().double(), vc.cpu().double()
+    for t in range(T):
+        pg, off = int(slots[t]) // page, int(slots[t]) % page
+        _close(kc_c[pg, :, off], want_k[t], dtype, scale=float(want_k.abs().max()))
+        _close(vc_c[pg, :, off], want_v[t], dtype, scale=float(want_v.abs().max()))
+    if rot == dh:
+        # the reference's form: adjacent pairs on row-permuted projections (scripts/jiuge.py:217-227)
+        perm = P.permute_rows_to_adjacent_pairs(torch.arange(dh, dtype=torch.float64)[:, None], 1, dh)[:, 0].long()
+        adj = P.plain_rope_adjacent(heads[:, :nh][..., perm], pos.tolist(), sin, cos)
+        _close(got[:, :nh][..., perm], adj, dtype)
+
+
+def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl):
+    """lens: list of (past, new) per request.  Returns (got, want) [T, nh*dh]."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(seed)
+    scale = 1.0 / math.sqrt(dh)
+    qs, want, token_req, positions, tables, kcs, vcs = [], [], [], [], [], [], []
+    page_base = 0
+    for r, (past, new) in enumerate(lens):
+        t = past + new
+        q = torch.randn(new, nh, dh, generator=g).to(dtype)
+        k = torch.randn(t, nkvh, dh, generator=g).to(dtype)
+        v = torch.randn(t, nkvh, dh, generator=g).to(dtype)
+        want.append(P.plain_attention(q, k, v, scale, past, window).reshape(new, nh * dh))
+        kc, vc, bt = _paged(k, v, page, dtype, seed=seed + r)
+        kcs.append(kc); vcs.append(vc)
+        tables.append(bt + page_base)
+        page_base += kc.shape[0]
+        qs.append(q.reshape(new, nh * dh))
+        token_req += [r] * new
+        positions += list(range(past, t))
+    maxb = max(len(b) for b in tables)
+    bt = torch.zeros(len(lens), maxb, dtype=torch.int32)
+    for r, b in enumerate(tables):
+        bt[r, :len(b)] = b
+    q = torch.cat(qs).to(DEV)
+    kc, vc = torch.cat(kcs).to(DEV), torch.cat(vcs).to(DEV)
+    out = torch.zeros_like(q)
+    T = q.shape[0]
+    tr = torch.tensor(token_req, dtype=torch.int32, device=DEV)
+    ps = torch.tensor(positions, dtype=torch.int32, device=DEV)
+    btd = bt.to(DEV)
+    if impl == "generic":
+        ops.attention_generic(q, out, kc, vc, btd, tr, ps, nh, nkvh, dh, page, scale, window or 0)
+    elif impl == "decode":
+        assert all(n == 1 for _, n in lens)
+        n_split = 3
+        pa = torch.empty(T * nh * n_split * dh, device=DEV)
+        pm = torch.empty(T * nh * n_split * 2, device=DEV)
+        ops.attention_decode(q, out, kc, vc, btd, None, T, tr, ps, pa, pm, nh, nkvh, dh, page, scale,
+                             window or 0, n_split)
+    else:
+        rows = ops.attention_prefill_tile_rows()
+        tiles, row0 = [], 0
+        for r, (past, new) in enumerate(lens):
+            for o in range(0, new, rows):
+                tiles += [r, row0 + o, min(rows, new - o), past + o]
+            row0 += new
+        tl = torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 4)
+        ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0)
+    return out, torch.cat(want)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("nh,nkvh,dh,page", [(4, 2, 16, 16), (3, 3, 32, 32), (5, 1, 48, 16), (6, 2, 64, 16),
+                                              (2, 1, 80, 64), (8, 2, 128, 64), (2, 2, 256, 16)])
+@pytest.mark.parametrize("window", [None, 37])
+def test_attention_generic(dtype, nh, nkvh, dh, page, window):
+    lens = [(0, 1), (0, 70), (130, 1), (64, 33), (15, 2), (257, 1)]
+    got, want = _attention_case(dtype, nh, nkvh, dh, page, lens, window, 11, "generic")
+    _close(got, want, dtype, factor=3)
+
+
+@pytest.mark.parametrize("dtype", DT)
+@pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (5, 1, 64, 32), (8, 2, 128, 16),
+                                              (16, 1, 128, 64)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_attention_decode(dtype, nh, nkvh, dh, page, window):
+    lens = [(0, 1), (1, 1), (63, 1), (64, 1), (700, 1), (255, 1), (1031, 1)]
+    got, want = _attention_case(dtype, nh, nkvh, dh, page, lens, window, 12, "decode")
+    _close(got, want, dtype, factor=3)
+
+
+@pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (3, 1, 64, 32), (4, 2, 128, 16),
+                                              (4, 4, 128, 64)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_attention_prefill_mfma(nh, nkvh, dh, page, window):
+    lens = [(0, 2), (0, 129), (130, 64), (64, 33), (15, 2), (257, 300), (5, 128)]
+    got, want = _attention_case(torch.bfloat16, nh, nkvh, dh, page, lens, window, 13, "prefill")
+    _close(got, want, torch.bfloat16, factor=3)
+
+
+def test_attention_special_cases():
+    """One key: the output is that value row.  Equal scores: the mean of the values.
+    No rotation, no mask (the last row of a prompt): the library's attention."""
+    dtype, nh, nkvh, dh, page = torch.float32, 2, 2, 32, 16
+    ops = _ops()
+    g = torch.Generator().manual_seed(14)
+    t = 40
+    k = torch.randn(t, nkvh, dh, generator=g)
+    v = torch.randn(t, nkvh, dh, generator=g)
+    q = torch.randn(t, nh, dh, generator=g)
+    kc, vc, bt = _paged(k, v, page, dtype)
+    tr = torch.zeros(t, dtype=torch.int32, device=DEV)
+    ps = torch.arange(t, dtype=torch.int32, device=DEV)
+    out = torch.empty(t, nh * dh, device=DEV)
+    scale = 1 / math.sqrt(dh)
+    ops.attention_generic(q.reshape(t, -1).to(DEV), out, kc.to(DEV), vc.to(DEV), bt[None].to(DEV), tr, ps,
+                          nh, nkvh, dh, page, scale, 0)
+    out = out.cpu().reshape(t, nh, dh)
+    _close(out[0], v[0], dtype)                                   # position 0 sees one key
+    lib = torch.nn.functional.scaled_dot_product_attention(
+        q.double().transpose(0, 1), k.double().transpose(0, 1), v.double().transpose(0, 1), is_causal=True)
+    _close(out, lib.transpose(0, 1), dtype, factor=5)
+    # equal scores: q = 0
+    out0 = torch.empty(t, nh * dh, device=DEV)
+    ops.attention_generic(torch.zeros(t, nh * dh, device=DEV), out0, kc.to(DEV), vc.to(DEV), bt[None].to(DEV),
+                          tr, ps, nh, nkvh, dh, page, scale, 0)
+    _close(out0.cpu().reshape(t, nh, dh)[-1], v.double().mean(0), dtype, factor=5)
+
+
+@pytest.mark.parametrize("impl,dtype", [("generic", torch.float32), ("generic", torch.bfloat16),
+                                        ("decode", torch.float32), ("decode", torch.bfloat16),
+                                        ("prefill", torch.bfloat16)])
+def test_attention_far_key_and_window_edge(impl, dtype):
+    """One far key among hundreds is made to stand out (its score dwarfs the rest):
+    the output must be its value row.  With a window, the key at its edge counts
+    and the key one step beyond does not."""
+    ops = _ops()
+    nh = nkvh = 2
+    dh, page = 64, 16
+    g = torch.Generator().manual_seed(15)
+    t = 777
+    past = t - 1 if impl != "prefill" else t - 150
+    new = t - past
+    scale = 1 / math.sqrt(dh)
+    for window, far, inside in [(None, 3, True), (None, 401, True), (300, t - 300, True), (300, t - 301, False)]:
+        k = torch.randn(t, nkvh, dh, generator=g) * 0.1
+        v = torch.randn(t, nkvh, dh, generator=g)
+        q = torch.randn(new, nh, dh, generator=g) * 0.1
+        k[far, :, 7] = 40.0
+        q[-1, :, 7] = 40.0            # the last query's score against key `far` is 1600/8 = 200
+        kc, vc, bt = _paged(k.to(dtype), v.to(dtype), page, dtype, seed=far)
+        kc, vc = kc.to(DEV), vc.to(DEV)
+        qd = q.to(dtype).reshape(new, -1).to(DEV)
+        out = torch.zeros(new, nh * dh, dtype=dtype, device=DEV)
+        tr = torch.zeros(new, dtype=torch.int32, device=DEV)
+        ps = torch.arange(past, t, dtype=torch.int32, device=DEV)
+        btd = bt[None].contiguous().to(DEV)
+        if impl == "generic":
+            ops.attention_generic(qd, out, kc, vc, btd, tr, ps, nh, nkvh, dh, page, scale, window or 0)
+        elif impl == "decode":
+            pa = torch.empty(nh * 4 * dh, device=DEV); pm = torch.empty(nh * 4 * 2, device=DEV)
+            ops.attention_decode(qd, out, kc, vc, btd, None, 1, tr, ps, pa, pm, nh, nkvh, dh, page, scale,
+                                 window or 0, 4)
+        else:
+            rows = ops.attention_prefill_tile_rows()
+            tiles = []
+            for o in range(0, new, rows):
+                tiles += [0, o, min(rows, new - o), past + o]
+            tl = torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 4)
+            ops.attention_prefill(qd, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0)
+        last = out[-1].float().cpu().reshape(nh, dh)
+        vfar = v[far].to(dtype).float()
+        hit = float((last - vfar).abs().max()) < 0.05
+        assert hit == inside, "window %s, key %d: expected %s" % (window, far, "seen" if inside else "not seen")
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("cdtype", DT)
+@pytest.mark.parametrize("M,N,K", [(1, 331, 200), (8, 2304, 2304), (16, 509, 96), (17, 1000, 344), (64, 777, 5760),
+                                   (3, 122753, 64), (130, 300, 100)])
+def test_gemm_nt(cdtype, M, N, K):
+    g = torch.Generator().manual_seed(16)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = torch.randn(N, K, generator=g).to(torch.bfloat16)
+    out = torch.empty(M, N, dtype=cdtype, device=DEV)
+    _ops().gemm_nt(a.to(DEV), w.to(DEV), out, 0.5)
+    want = 0.5 * P.plain_linear(a, w)
+    _close(out, want, cdtype, factor=2)
+
+
+def test_library_float32_product_is_true_float32():
+    """The float32 path's matrix products must not run in a reduced-precision mode."""
+    from infinicore_infer_amd.parts.linear import linear
+    g = torch.Generator().manual_seed(17)
+    a = torch.randn(200, 2304, generator=g)
+    w = torch.randn(500, 2304, generator=g)
+    out = torch.empty(200, 500, device=DEV)
+    linear(a.to(DEV), w.to(DEV), out)
+    want = a.double() @ w.double().t()
+    err = float((out.cpu().double() - want).abs().max()) / float(want.abs().max())
+    assert err < 5e-6, "float32 product error %.3g: a reduced-precision mode is on" % err
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("V", [256, 509, 122753])
+def test_sampling(V):
+    ops = _ops()
+    g = torch.Generator().manual_seed(18)
+    cases = [(0.0, 0, 1.0), (1.0, 1, 1.0), (1.0, 0, 1.0), (0.7, 5, 1.0), (1.3, 0, 0.8), (0.9, 40, 0.6),
+             (2.0, V, 0.95), (1.0, 3, 0.01)]
+    R = len(cases) * 6
+    logits = torch.randn(R, V, generator=g) * 3
+    logits[0, 10] = logits[0, 20] = 50.0                  # equal maxima: the lowest index wins
+    temps = torch.tensor([c[0] for c in cases] * 6)
+    ks = torch.tensor([c[1] for c in cases] * 6, dtype=torch.int32)
+    ps = torch.tensor([c[2] for c in cases] * 6)
+    us = torch.rand(R, generator=g)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), out, temps.to(DEV), ks.to(DEV), ps.to(DEV), us.to(DEV))
+    got = out.cpu().tolist()
+    assert got[0] == 10
+    for r in range(R):
+        want = P.plain_sample(logits[r], float(temps[r]), int(ks[r]), float(ps[r]), float(us[r]))
+        assert got[r] == want, "row %d (T=%g k=%d p=%g u=%g): got %d, plain %d" % (
+            r, temps[r], ks[r], ps[r], us[r], got[r], want)
+    # argmax for every row when no temperature is given
+    ops.sample(logits.to(DEV), out)
+    assert out.cpu().tolist() == [int(torch.argmax(logits[r])) for r in range(R)]
+
+
+def test_sampling_distribution():
+    """Many draws at temperature 1 follow softmax (chi-square against torch.softmax)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(19)
+    V, n = 12, 20000
+    row = torch.randn(V, generator=g)
+    logits = row[None].expand(n, V).contiguous().to(DEV)
+    us = torch.rand(n, generator=g).to(DEV)
+    out = torch.empty(n, dtype=torch.int32, device=DEV)
+    ops.sample(logits, out, torch.ones(n, device=DEV), torch.zeros(n, dtype=torch.int32, device=DEV),
+               torch.ones(n, device=DEV), us)
+    counts = torch.bincount(out.cpu().long(), minlength=V).double()
+    expect = torch.softmax(row.double(), 0) * n
+    chi2 = float(((counts - expect) ** 2 / expect).sum())
+    assert chi2 < 40.0, "chi-square %.1f over %d bins" % (chi2, V)       # 11 dof: p(chi2 > 40) < 1e-4
