@@ -1,0 +1,171 @@
+#!/usr/bin/python3
+"""Decode and prefill throughput of the MiniCPM-2B-shaped model on one MI355X.
+
+  python bench.py --gpus 1 --steps K --warmup W
+
+A step is one decode step of the whole batch: the step function over one new
+token per request, greedy sampling on the device, and the sampled tokens fed
+back (the reference times the same loop, scripts/jiuge.py:562-583, prefill
+excluded).  Weights are random (seeded), prompts are seeded uniform-random token
+ids.  One JSON line is printed.
+"""
+import argparse
+import json
+import math
+import sys
+import time
+
+import torch
+
+HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
+PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
+
+# BASELINE.json configs[2]: MiniCPM-2B-shaped
+MODEL = dict(
+    model_type="minicpm", vocab_size=122753, hidden_size=2304, num_hidden_layers=40,
+    num_attention_heads=36, num_key_value_heads=36, intermediate_size=5760,
+    max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0,
+    scale_emb=12, dim_model_base=256, scale_depth=1.4, tie_word_embeddings=True, eos_token_id=2)
+PROMPT = 2048
+BATCH = 8
+WEIGHT_STD = 0.1
+
+
+def _sync():
+    torch.cuda.synchronize()
+
+
+def build_engine(layers, max_tokens, max_requests, page_size):
+    from infinicore_infer_amd.config import config_from_dict
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.parts import Runtime, build_model
+    from infinicore_infer_amd.weights import init_random_weights
+    cfg = dict(MODEL, num_hidden_layers=layers)
+    conf = config_from_dict(cfg)
+    model = build_model(conf.model_spec(), Runtime(dtype=torch.bfloat16, device="cuda:0"))
+    init_random_weights(model, seed=0, std=WEIGHT_STD, tie=True)
+    return Engine(model, max_tokens=max_tokens, page_size=page_size, max_requests=max_requests), conf
+
+
+def model_numbers(conf):
+    """Bytes of weights a decode step reads once, cache bytes per token, flops per prefill."""
+    d, L, di, V = conf.hidden_size, conf.num_hidden_layers, conf.intermediate_size, conf.vocab_size
+    nh, nkvh, dh = conf.num_attention_heads, conf.num_key_value_heads, conf.head_dim
+    per_layer = (nh + 2 * nkvh) * dh * d + nh * dh * d + 3 * d * di
+    weight_bytes = 2 * (L * per_layer + V * d) + 4 * d * (2 * L + 1)
+    kv_bytes_per_token = 2 * L * nkvh * dh * 2
+
+    def prefill_flops(T):
+        linear = 2.0 * T * L * per_layer
+        attn = L * nh * dh * 4.0 * (T * (T + 1) / 2)        # QK^T and PV over the causal half
+        head = 2.0 * V * d                                   # last row only
+        return linear + attn + head
+    return weight_bytes, kv_bytes_per_token, prefill_flops
+
+
+def time_prefill(engine, tokens, reps=3):
+    from infinicore_infer_amd.engine import StepEntry
+    best = None
+    for i in range(reps + 1):
+        _sync()
+        t0 = time.perf_counter()
+        logits = engine.step([StepEntry("pf", tokens, [len(tokens) - 1])])
+        engine.sample(logits)
+        _sync()
+        dt = time.perf_counter() - t0
+        engine.free("pf")
+        if i > 0:
+            best = dt if best is None else min(best, dt)
+    return best
+
+
+def time_decode(engine, batch, steps, warmup, vocab, seed=0):
+    """Prefill ``batch`` requests of PROMPT tokens, then time ``steps`` decode steps."""
+    from infinicore_infer_amd.engine import StepEntry
+    g = torch.Generator().manual_seed(seed)
+    ids = ["d%d" % i for i in range(batch)]
+    last = []
+    for rid in ids:
+        toks = torch.randint(0, vocab, (PROMPT,), generator=g).tolist()
+        logits = engine.step([StepEntry(rid, toks, [PROMPT - 1])])
+        last.append(engine.sample(logits)[0])
+
+    def one():
+        nonlocal last
+        logits = engine.step([StepEntry(rid, [t], [0]) for rid, t in zip(ids, last)])
+        last = engine.sample(logits)
+
+    for _ in range(warmup):
+        one()
+    _sync()
+    ctx0 = engine.length(ids[0])
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        one()
+    _sync()
+    dt = time.perf_counter() - t0
+    ctx1 = engine.length(ids[0])
+    for rid in ids:
+        engine.free(rid)
+    return dt / steps, (ctx0 + ctx1) / 2.0
+
+
+def main():
+    ap = argparse.ArgumentParser()
+    ap.add_argument("--gpus", type=int, default=1)
+    ap.add_argument("--steps", type=int, default=128)
+    ap.add_argument("--warmup", type=int, default=16)
+    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
+    ap.add_argument("--page-size", type=int, default=64)
+    ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    args = ap.parse_args()
+    if args.gpus != 1:
+        print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
+        return 2
+
+    sys.path.insert(0, __import__("os").path.dirname(__import__("os").path.abspath(__file__)))
+    per_req = PROMPT + args.warmup + args.steps + 64
+    per_req = (per_req + 63) // 64 * 64
+    batches = [BATCH] if args.no_points else [BATCH, 1, 64]
+    engine, conf = build_engine(args.layers, per_req * max(batches), max(batches) + 1, args.page_size)
+    weight_bytes, kv_per_tok, prefill_flops = model_numbers(conf)
+    vocab = conf.vocab_size
+
+    g = torch.Generator().manual_seed(123)
+    ptoks = torch.randint(0, vocab, (PROMPT,), generator=g).tolist()
+    t_pf = time_prefill(engine, ptoks)
+    pf_flops = prefill_flops(PROMPT)
+
+    results = {}
+    for b in batches:
+        results[b] = time_decode(engine, b, args.steps, args.warmup, vocab, seed=b)
+    ms, ctx = results[BATCH][0] * 1e3, results[BATCH][1]
+    value = BATCH / results[BATCH][0]
+    bytes_step = weight_bytes + BATCH * ctx * kv_per_tok
+    achieved = bytes_step / results[BATCH][0] / 1e9
+
+    out = {
+        "metric": "decode tokens/s, batch 8, 2048-token prompts (MiniCPM-2B-shaped)",
+        "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
+        "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (seeded random weights N(0,0.1) and token ids)",
+        "config": {
+            "model": "MiniCPM-2B-shaped", "layers": conf.num_hidden_layers, "layers_of_config": MODEL["num_hidden_layers"],
+            "hidden": conf.hidden_size, "heads": conf.num_attention_heads, "kv_heads": conf.num_key_value_heads,
+            "head_dim": conf.head_dim, "intermediate": conf.intermediate_size, "vocab": conf.vocab_size,
+            "global_batch": BATCH, "seq_len": PROMPT, "context_mean": round(ctx, 1), "generated": args.steps,
+            "page_size": args.page_size, "tied_embeddings": True, "parallelism": "single-gpu",
+            "sampling": "greedy on device",
+        },
+        "prefill": {"value": round(PROMPT / t_pf, 1), "tokens": PROMPT, "ms": round(t_pf * 1e3, 3),
+                    "frac": round(pf_flops / t_pf / (PEAK_TFLOPS["bf16"] * 1e12), 4)},
+        "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                     "frac": round(achieved / HBM_PEAK_GBS, 4)},
+        "points": {("decode_b%d" % b): round(b / results[b][0], 1) for b in batches if b != BATCH},
+    }
+    print(json.dumps(out))
+    return 0
+
+
+if __name__ == "__main__":
+    sys.exit(main())

@@ -51,6 +51,28 @@ def random_state_dict(config: dict, seed: int, std: float = 0.02, norm_std: floa
     return out
 
 
+def init_random_weights(model, seed: int, std: float = 0.02, norm_std: float = 0.0, tie: bool = True) -> None:
+    """Random weights straight into a built model, drawn on the model's device
+    (no folder is written).  Same rules as ``random_state_dict``; matrices are
+    rounded to the model's compute dtype, norm weights stay float32."""
+    rt = model.runtime
+    specs = model.weight_specs()
+    tensors: Dict[str, torch.Tensor] = {}
+    for name, spec in specs.items():
+        if tie and spec.fallback in specs and spec.fallback in tensors:
+            tensors[name] = tensors[spec.fallback]
+            continue
+        g = _generator(seed, name, rt.device)
+        if spec.role == "vector":
+            t = torch.ones(spec.shape, dtype=torch.float32, device=rt.device)
+            if norm_std:
+                t = t + norm_std * torch.randn(spec.shape, generator=g, dtype=torch.float32, device=rt.device)
+        else:
+            t = (std * torch.randn(spec.shape, generator=g, dtype=torch.float32, device=rt.device)).to(rt.dtype)
+        tensors[name] = t
+    model.load_weights(tensors)
+
+
 def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, norm_std: float = 0.0,
                        dtype: torch.dtype = torch.bfloat16) -> str:
     """Write config.json and model.safetensors into ``folder``; returns it."""
