@@ -1,0 +1,238 @@
+"""The scheduler above the step function: admits requests, cuts prompts into
+portions under a token budget, decodes, finishes and frees.
+
+The reference's only scheduler is the server's worker loop
+(scripts/launch_server.py:134-159): it pops up to MAX_BATCH tasks, runs one
+inferBatch over them (a new task's whole prompt beside the others' single
+tokens), re-queues the unfinished ones and releases the finished ones' caches;
+there is no token budget and memory is committed per whole-context slab
+(scripts/kvcache_pool.py:18-42).  Here:
+
+  * waiting requests are admitted first come first served while a state slot is
+    free and the pages of their first portion are there;
+  * every step takes all running requests that decode (one token each) first,
+    then prompt portions of at most ``chunk_size`` tokens until
+    ``max_batch_tokens`` are spent;
+  * when pages run out for a decode token, the most recently admitted running
+    request is preempted: its pages and slot are given back and it returns to
+    the FRONT of the waiting queue with prompt + generated tokens to be
+    recomputed; its random draws depend only on (seed, id, token index), so the
+    continuation is the same.  A request that cannot fit even alone finishes
+    with finish_reason "length".
+
+The scheduler only needs ``engine.cache`` (a CacheManager), ``engine.step``,
+``engine.sample``, ``engine.add_request`` and ``engine.free``, so its decisions
+are tested on the CPU with a stand-in engine.
+"""
+from collections import deque
+from dataclasses import dataclass, field
+from typing import Deque, Dict, List, Optional, Tuple
+
+from ..cache import OutOfPages
+from ..sampling import uniform_draw
+from .engine import StepEntry
+from .tasks import InferTask
+
+
+@dataclass
+class _Running:
+    task: InferTask
+    feed: List[int]                  # tokens of this request still to be computed (prompt, or prompt + generated)
+    cursor: int = 0                  # how many of ``feed`` are computed
+    order: int = 0                   # admission counter (larger = admitted later)
+
+    @property
+    def decoding(self) -> bool:
+        return self.cursor >= len(self.feed)
+
+
+class Scheduler:
+    def __init__(self, engine, max_batch_tokens: int = 2048, chunk_size: int = 512,
+                 max_running: Optional[int] = None):
+        if max_batch_tokens < 1 or chunk_size < 1:
+            raise ValueError("max_batch_tokens and chunk_size must be positive")
+        self.engine = engine
+        self.cache = engine.cache
+        self.max_batch_tokens = max_batch_tokens
+        self.chunk_size = chunk_size
+        self.max_running = max_running or self.cache.max_requests
+        self.waiting: Deque[_Running] = deque()
+        self.running: List[_Running] = []
+        self.finished: List[InferTask] = []
+        self._admitted = 0
+        self.n_preempted = 0
+        self.n_steps = 0
+        self.last_plan: List[Tuple[object, int, int]] = []     # (id, first position, tokens) of the last step
+
+    # ---- queueing -----------------------------------------------------------------
+    def add(self, task: InferTask) -> None:
+        if not task.prompt:
+            raise ValueError("request %r has an empty prompt" % (task.id,))
+        self.waiting.append(_Running(task, list(task.prompt)))
+
+    def has_unfinished(self) -> bool:
+        return bool(self.waiting or self.running)
+
+    def abort(self, task_id) -> None:
+        for r in list(self.running):
+            if r.task.id == task_id:
+                self._finish(r, "cancel")
+        for r in list(self.waiting):
+            if r.task.id == task_id:
+                self.waiting.remove(r)
+                r.task.finish_reason = "cancel"
+                self.finished.append(r.task)
+
+    # ---- internals --------------------------------------------------------------------
+    def _finish(self, r: _Running, reason: str) -> None:
+        r.task.finish_reason = reason
+        self.engine.free(r.task.id)
+        if r in self.running:
+            self.running.remove(r)
+        self.finished.append(r.task)
+
+    def _preempt(self, r: _Running) -> None:
+        """Give back everything ``r`` holds; it will be recomputed from its tokens."""
+        self.engine.free(r.task.id)
+        self.running.remove(r)
+        r.feed = list(r.task.prompt) + list(r.task.generated)
+        r.cursor = 0
+        self.waiting.appendleft(r)
+        self.n_preempted += 1
+
+    def _pages_for_new(self, n_tokens: int) -> List[int]:
+        ps = self.cache.page_size
+        return [(n_tokens + ps - 1) // ps] * len(self.cache.groups)
+
+    def _fits(self, need: List[int], reserved: List[int]) -> bool:
+        return all(n + r <= self.cache.free_pages(g) for g, (n, r) in enumerate(zip(need, reserved)))
+
+    # ---- one step -------------------------------------------------------------------------
+    def plan(self) -> List[Tuple[_Running, int]]:
+        """Decide which request computes how many tokens in the next step."""
+        ngroups = len(self.cache.groups)
+        reserved = [0] * ngroups
+        budget = self.max_batch_tokens
+        plan: List[Tuple[_Running, int]] = []
+
+        # 1. decodes, oldest first; preempt the youngest when pages run out
+        for r in sorted([r for r in self.running if r.decoding], key=lambda r: r.order):
+            if r not in self.running or budget < 1:
+                continue
+            while True:
+                need = self.cache.pages_needed(r.task.id, 1)
+                if self._fits(need, reserved):
+                    reserved = [a + b for a, b in zip(reserved, need)]
+                    plan.append((r, 1))
+                    budget -= 1
+                    break
+                victim = max(self.running, key=lambda x: x.order)
+                planned = [p for p in plan if p[0] is victim]
+                if planned:                      # a younger request already has its page this step: take it back
+                    plan.remove(planned[0])
+                    budget += planned[0][1]
+                    back = self.cache.pages_needed(victim.task.id, planned[0][1])
+                    reserved = [a - b for a, b in zip(reserved, back)]
+                if victim is r and len(self.running) == 1:
+                    self._finish(r, "length")        # alone and still no room: the cache is too small for it
+                    break
+                self._preempt(victim)
+                if victim is r:
+                    break
+
+        # 2. prompt portions of running requests, oldest first
+        for r in sorted([r for r in self.running if not r.decoding], key=lambda r: r.order):
+            if budget < 1:
+                break
+            n = min(self.chunk_size, len(r.feed) - r.cursor, budget)
+            need = self.cache.pages_needed(r.task.id, n)
+            if not self._fits(need, reserved):
+                continue
+            reserved = [a + b for a, b in zip(reserved, need)]
+            plan.append((r, n))
+            budget -= n
+
+        # 3. admissions, first come first served
+        while self.waiting and budget >= 1 and len(self.running) < self.max_running \
+                and self.cache.slots.n_free > 0:
+            r = self.waiting[0]
+            if self.cache.max_positions is not None and len(r.feed) > self.cache.max_positions:
+                self.waiting.popleft()
+                r.task.finish_reason = "length"
+                self.finished.append(r.task)
+                continue
+            n = min(self.chunk_size, len(r.feed), budget)
+            need = self._pages_for_new(n)
+            if not self._fits(need, reserved):
+                break
+            self.waiting.popleft()
+            self.engine.add_request(r.task.id)
+            self._admitted += 1
+            r.order = self._admitted
+            self.running.append(r)
+            reserved = [a + b for a, b in zip(reserved, need)]
+            plan.append((r, n))
+            budget -= n
+
+        # nothing can move although requests run: make room by preempting the youngest
+        if not plan and self.running:
+            victim = max(self.running, key=lambda x: x.order)
+            if len(self.running) == 1:
+                self._finish(victim, "length")
+            else:
+                self._preempt(victim)
+            return self.plan()
+        if not plan and self.waiting and not self.running:
+            r = self.waiting.popleft()               # does not fit an empty cache
+            r.task.finish_reason = "length"
+            self.finished.append(r.task)
+            return self.plan()
+        return plan
+
+    def step(self) -> List[Tuple[InferTask, int]]:
+        """Run one step; returns (task, new token) for every request that got a token."""
+        plan = self.plan()
+        if not plan:
+            return []
+        entries, samplers = [], []
+        self.last_plan = []
+        for r, n in plan:
+            toks = r.feed[r.cursor:r.cursor + n] if not r.decoding else [r.task.generated[-1]]
+            last = r.decoding or r.cursor + n == len(r.feed)
+            entries.append(StepEntry(r.task.id, toks, [len(toks) - 1] if last else []))
+            self.last_plan.append((r.task.id, self.cache.length(r.task.id), len(toks)))
+            if last:
+                samplers.append(r)
+        logits = self.engine.step(entries)
+        for r, n in plan:
+            if not r.decoding:
+                r.cursor += n
+        self.n_steps += 1
+        out: List[Tuple[InferTask, int]] = []
+        if samplers:
+            tasks = [r.task for r in samplers]
+            if all(t.temperature == 0 or t.topk == 1 for t in tasks):
+                tokens = self.engine.sample(logits)
+            else:
+                tokens = self.engine.sample(
+                    logits, [t.temperature for t in tasks], [t.topk for t in tasks], [t.topp for t in tasks],
+                    [uniform_draw(t.seed, t.id, len(t.generated)) for t in tasks])
+            for r, tok in zip(samplers, tokens):
+                t = r.task
+                t.generated.append(int(tok))
+                t.pos = self.cache.length(t.id)
+                out.append((t, int(tok)))
+                if tok in t.end_tokens:
+                    self._finish(r, "stop")
+                elif t.pos >= t.max_tokens:
+                    self._finish(r, "length")
+                elif t.max_new_tokens is not None and len(t.generated) >= t.max_new_tokens:
+                    self._finish(r, "length")
+        return out
+
+    def run(self) -> List[InferTask]:
+        """Step until every request has finished."""
+        while self.has_unfinished():
+            self.step()
+        done, self.finished = self.finished, []
+        return done

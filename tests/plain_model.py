@@ -160,7 +160,7 @@ def plain_swiglu(gate, up):
 # --------------------------------------------------------------------------
 # whole model                                  src/models/jiuge/jiuge.cpp:195-267
 # --------------------------------------------------------------------------
-def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", window=None):
+def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", window=None, start_pos=0):
     """Logits [T, vocab] (float64) of one request's whole token sequence from
     position 0.  ``weights``: tensors by checkpoint name (jiuge.py:33-77)."""
     rnd = rnd or _ident
@@ -170,9 +170,9 @@ def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", 
     theta = cfg.get("rope_theta", 100000.0)                       # jiuge.py:133
     s_in, s_out, s_res = plain_scales(cfg, logit_scale_rule)
     T = len(tokens)
-    positions = list(range(T))
+    positions = list(range(start_pos, start_pos + T))     # start_pos != 0 only to test that distances alone count
     factors, magnitude = plain_longrope(cfg)
-    sin, cos = plain_rope_tables(dh, theta, T, factors, magnitude)
+    sin, cos = plain_rope_tables(dh, theta, start_pos + T, factors, magnitude)
 
     emb_name = "model.embed_tokens.weight"
     head_name = "lm_head.weight"
@@ -211,8 +211,8 @@ def plain_sample(logits, temperature, top_k, top_p, u):
     temperature, keep every value >= the k-th largest (k = 0 or k >= V keeps
     all), softmax, keep the most probable tokens up to and including the one
     with which the kept mass reaches top_p (equal values are kept together),
-    then walk the kept tokens in vocabulary order and return the first whose
-    cumulated mass reaches u * total."""
+    then walk the kept tokens in vocabulary order and return the first (of
+    non-zero mass) whose cumulated mass reaches u * total."""
     z = torch.as_tensor(logits, dtype=F64)
     V = z.numel()
     if temperature == 0 or top_k == 1:
@@ -234,7 +234,7 @@ def plain_sample(logits, temperature, top_k, top_p, u):
         total = p.sum()
     target = u * total
     csum = torch.cumsum(p, 0)
-    cand = torch.nonzero((csum >= target) & keep)
+    cand = torch.nonzero((csum >= target) & keep & (p > 0))
     if cand.numel() == 0:
         return int(torch.nonzero(keep)[-1])
     return int(cand[0])

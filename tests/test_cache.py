@@ -1,0 +1,99 @@
+"""The cache manager: no page lost, held twice or freed twice, under random orders of requests (CPU)."""
+import random
+
+import pytest
+
+from infinicore_infer_amd.cache import (CacheError, CacheManager, GroupSpec, OutOfPages, PagePool,
+                                        PositionOverflow)
+
+FULL = GroupSpec("full", 2, 16, None, (0, 1))
+WIN = GroupSpec("window", 2, 16, 40, (2,))
+
+
+def test_pool_basics_and_double_free():
+    p = PagePool(3)
+    a, b, c = p.alloc(), p.alloc(), p.alloc()
+    assert sorted([a, b, c]) == [0, 1, 2] and p.n_free == 0
+    with pytest.raises(OutOfPages):
+        p.alloc()
+    p.free(b)
+    assert p.alloc() == b                      # last freed, first reused
+    p.free(a)
+    with pytest.raises(CacheError):
+        p.free(a)
+    with pytest.raises(CacheError):
+        p.free(7)
+
+
+def test_append_block_tables_and_slots():
+    m = CacheManager([FULL], 8, 16, max_requests=2, max_positions=100)
+    m.admit("a")
+    assert m.append("a", 17) == 0
+    assert len(m.block_table("a", 0)) == 2 and m.length("a") == 17
+    assert m.append("a", 15) == 17 and len(m.block_table("a", 0)) == 2
+    assert m.append("a", 1) == 32 and len(m.block_table("a", 0)) == 3
+    t = m.block_table("a", 0)
+    assert m.slot_of("a", 0, 16) == t[1] * 16 and m.slot_of("a", 0, 32) == t[2] * 16
+    with pytest.raises(PositionOverflow):
+        m.append("a", 100)
+    m.admit("b")
+    with pytest.raises(OutOfPages):
+        m.admit("c")
+    with pytest.raises(OutOfPages):
+        m.append("b", 16 * 6)                    # 5 pages left
+    assert m.length("b") == 0 and m.free_pages() == 5
+    assert not m.can_append("b", 16 * 5, reserve=[1]) and m.can_append("b", 16 * 5)
+    m.release("a")
+    m.release("b")
+    assert m.free_pages() == 8 and m.slots.n_free == 2
+    m.check_invariants()
+
+
+def test_window_group_gives_pages_back_early():
+    m = CacheManager([FULL, WIN], [16, 16], 16, max_requests=2)
+    m.admit("a")
+    m.append("a", 100)
+    assert m.trim("a") == 3                      # next query 100 reads keys >= 61: pages 0..2 are dead
+    assert m.block_table("a", 1)[:4] == [-1, -1, -1, m.block_table("a", 1)[3]]
+    assert m.free_pages(1) == 16 - 7 + 3 and m.free_pages(0) == 16 - 7
+    with pytest.raises(CacheError):
+        m.slot_of("a", 1, 5)
+    m.append("a", 28)
+    assert m.trim("a") == 2                      # next query 128 reads keys >= 89: pages 3, 4 go too
+    assert m.trim("a") == 0
+    m.check_invariants()
+    m.release("a")
+    assert m.free_pages(0) == 16 and m.free_pages(1) == 16
+    m.check_invariants()
+
+
+@pytest.mark.parametrize("seed", range(8))
+def test_random_orders_conserve_pages(seed):
+    rng = random.Random(seed)
+    m = CacheManager([FULL, WIN], [24, 24], 16, max_requests=5, max_positions=400)
+    live, n = [], 0
+    for _ in range(600):
+        op = rng.random()
+        if op < 0.25 and m.can_admit():
+            n += 1
+            m.admit(n)
+            live.append(n)
+        elif op < 0.8 and live:
+            r = rng.choice(live)
+            k = rng.choice([1, 1, 1, 2, 7, 16, 33])
+            try:
+                m.append(r, k)
+                m.trim(r)
+            except (OutOfPages, PositionOverflow):
+                before = (m.length(r), m.free_pages(0), m.free_pages(1))
+                assert before == (m.length(r), m.free_pages(0), m.free_pages(1))
+        elif live:
+            r = live.pop(rng.randrange(len(live)))
+            m.release(r)
+            with pytest.raises(KeyError):
+                m.release(r)
+        m.check_invariants()
+    for r in live:
+        m.release(r)
+    m.check_invariants()
+    assert m.free_pages(0) == 24 and m.free_pages(1) == 24 and m.slots.n_free == 5

@@ -1,0 +1,373 @@
+"""Each part alone against its plain function; greedy generation through the entry point and
+the scheduler; and a toy architecture defined HERE (a mixer with state of its own, a windowed
+attention layer, a layer that reads another layer's cache, a layer run twice) that is registered,
+built and stepped without a change to the framework's files."""
+import math
+
+import pytest
+import torch
+
+import helpers as H
+import plain_model as P
+
+pytestmark = pytest.mark.gpu
+DEV = "cuda:0"
+
+
+# ---------------------------------------------------------------------------
+# a hand-made step context: one or more requests, identity page mapping
+# ---------------------------------------------------------------------------
+def _context(lens, page_size, n_kv_heads, head_dim, dtype, n_slots=1):
+    """lens: list of (past, new).  Pages are laid out one request after the other."""
+    from infinicore_infer_amd.engine.context import LayerCacheView, StepContext, Workspace
+    ctx = StepContext()
+    positions, token_req, slots, tables, dec, tiles = [], [], [], [], [], []
+    page0, row0 = 0, 0
+    maxb = max((p + n + page_size - 1) // page_size for p, n in lens)
+    for r, (past, new) in enumerate(lens):
+        nb = (past + new + page_size - 1) // page_size
+        tables.append(list(range(page0, page0 + nb)) + [0] * (maxb - nb))
+        for p in range(past, past + new):
+            positions.append(p)
+            token_req.append(r)
+            slots.append((page0 + p // page_size) * page_size + p % page_size)
+        if new == 1:
+            dec.append(row0)
+        else:
+            for o in range(0, new, 128):
+                tiles += [r, row0 + o, min(128, new - o), past + o]
+        page0 += nb
+        row0 += new
+    i32 = lambda v: torch.tensor(v, dtype=torch.int32, device=DEV)
+    ctx.T, ctx.R, ctx.page_size, ctx.ws = row0, len(lens), page_size, Workspace(DEV)
+    ctx.positions, ctx.token_req = i32(positions), i32(token_req)
+    ctx.decode_rows, ctx.n_decode_rows = i32(dec), len(dec)
+    ctx.decode_rows_identity = len(dec) == row0
+    ctx.prefill_tiles, ctx.n_prefill_tiles = i32(tiles).view(-1, 4), len(tiles) // 4
+    ctx.max_position = max(positions)
+    ctx.max_context = max(positions) + 1
+    views = []
+    for _ in range(n_slots):
+        k = torch.zeros(page0, n_kv_heads, page_size, head_dim, dtype=dtype, device=DEV)
+        views.append(LayerCacheView(k=k, v=torch.zeros_like(k), slots=i32(slots),
+                                    block_tables=i32(tables).view(len(lens), maxb)))
+    return ctx, views
+
+
+def _rel(got, want):
+    got, want = got.double().cpu(), want.double().cpu()
+    return float((got - want).abs().max()) / float(want.abs().max())
+
+
+DT = [(torch.float32, 2e-5), (torch.bfloat16, 2e-2)]
+
+
+@pytest.mark.parametrize("dtype,tol", DT)
+def test_norm_part(dtype, tol):
+    from infinicore_infer_amd.parts import Runtime, build_part
+    from infinicore_infer_amd.config import PartSpec
+    rt = Runtime(dtype, DEV)
+    norm = build_part("norm", PartSpec("rmsnorm", "n.", {"size": 200, "eps": 1e-6}), rt)
+    assert list(norm.weight_specs()) == ["n.weight"]
+    w = 1 + 0.2 * torch.randn(200)
+    norm.load_weights({"n.weight": w.to(DEV)})
+    x = torch.randn(9, 200)
+    y = torch.randn(9, 200).to(dtype)
+    out = torch.empty(9, 200, dtype=dtype, device=DEV)
+    norm.forward(x.to(DEV), out)
+    assert _rel(out, P.plain_rmsnorm(x, w, 1e-6)) < tol
+    xd = x.to(DEV).clone()
+    norm.forward_add(xd, y.to(DEV), 0.5, out)
+    assert _rel(out, P.plain_rmsnorm(x.double() + 0.5 * y.double(), w, 1e-6)) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", DT)
+def test_feed_forward_part(dtype, tol):
+    from infinicore_infer_amd.parts import Runtime, build_part
+    from infinicore_infer_amd.config import PartSpec
+    rt = Runtime(dtype, DEV)
+    ffn = build_part("feed_forward", PartSpec("swiglu", "m.", {"hidden_size": 72, "intermediate_size": 200}), rt)
+    w = {"m.gate_proj.weight": torch.randn(200, 72) * 0.1, "m.up_proj.weight": torch.randn(200, 72) * 0.1,
+         "m.down_proj.weight": torch.randn(72, 200) * 0.1}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    assert set(ffn.weight_specs()) == set(w)
+    ffn.load_weights({k: v.to(DEV) for k, v in w.items()})
+    ctx, _ = _context([(0, 11)], 16, 1, 16, dtype)
+    h = torch.randn(11, 72).to(dtype)
+    rnd = P.round_bf16 if dtype == torch.bfloat16 else (lambda t: t)
+    act = rnd(P.plain_swiglu(rnd(P.plain_linear(h, w["m.gate_proj.weight"])), rnd(P.plain_linear(h, w["m.up_proj.weight"]))))
+    want = P.plain_linear(act, w["m.down_proj.weight"])
+    assert _rel(ffn.forward(h.to(DEV), ctx), want) < tol
+
+
+@pytest.mark.parametrize("dtype,tol", DT)
+@pytest.mark.parametrize("nh,nkvh,dh,window,scaling", [(4, 2, 16, None, None), (6, 2, 64, None, "long"),
+                                                        (3, 3, 32, 20, None), (2, 1, 128, None, "short")])
+def test_attention_and_rotary_parts(dtype, tol, nh, nkvh, dh, window, scaling):
+    """The attention mixer (projection, rotary part, cache write, attention kernels, output
+    projection) on a prompt portion with a past, and on single tokens, against the plain
+    functions on the reference's permuted weights."""
+    from infinicore_infer_amd.parts import Runtime, build_part
+    from infinicore_infer_amd.config import PartSpec
+    rt = Runtime(dtype, DEV)
+    d, max_pos = 88, 256
+    sc = None
+    if scaling:
+        sc = dict(type="longrope", original_max_position_embeddings=64 if scaling == "long" else 512,
+                  short_factor=[1 + 0.1 * i for i in range(dh // 2)], long_factor=[2 + 0.1 * i for i in range(dh // 2)])
+    rot = PartSpec("rotary", "", {"head_dim": dh, "theta": 5000.0, "max_positions": max_pos, "scaling": sc})
+    att = build_part("mixer", PartSpec("attention", "a.", {
+        "hidden_size": d, "num_heads": nh, "num_kv_heads": nkvh, "head_dim": dh,
+        "softmax_scale": 1 / math.sqrt(dh), "window": window, "position_encoding": rot}), rt)
+    g = torch.Generator().manual_seed(dh)
+    w = {"a.q_proj.weight": torch.randn(nh * dh, d, generator=g) * 0.2, "a.k_proj.weight": torch.randn(nkvh * dh, d, generator=g) * 0.2,
+         "a.v_proj.weight": torch.randn(nkvh * dh, d, generator=g) * 0.2, "a.o_proj.weight": torch.randn(d, nh * dh, generator=g) * 0.2}
+    w = {k: v.to(dtype) for k, v in w.items()}
+    att.load_weights({k: v.to(DEV) for k, v in w.items()})
+    need = att.cache_need()
+    assert (need.kind, need.n_kv_heads, need.head_dim, need.window) == ("kv", nkvh, dh, window)
+
+    total, cut = 150, 97
+    h = torch.randn(total, d, generator=g).to(dtype)
+    rnd = P.round_bf16 if dtype == torch.bfloat16 else (lambda t: t)
+    cfg = {"rope_scaling": sc, "max_position_embeddings": max_pos}
+    factors, mag = P.plain_longrope(cfg)
+    sin, cos = P.plain_rope_tables(dh, 5000.0, total, factors, mag)
+    q = rnd(P.plain_linear(h, P.permute_rows_to_adjacent_pairs(w["a.q_proj.weight"].double(), nh, dh))).reshape(total, nh, dh)
+    k = rnd(P.plain_linear(h, P.permute_rows_to_adjacent_pairs(w["a.k_proj.weight"].double(), nkvh, dh))).reshape(total, nkvh, dh)
+    v = rnd(P.plain_linear(h, w["a.v_proj.weight"])).reshape(total, nkvh, dh)
+    q = rnd(P.plain_rope_adjacent(q, range(total), sin, cos))
+    k = rnd(P.plain_rope_adjacent(k, range(total), sin, cos))
+    a = rnd(P.plain_attention(q, k, v, 1 / math.sqrt(dh), 0, window)).reshape(total, nh * dh)
+    want = P.plain_linear(a, w["a.o_proj.weight"])
+
+    # one cache for the whole test: first portion, second portion with a past, then single tokens
+    ctx_all, views = _context([(0, total)], 16, nkvh, dh, dtype)
+    view = views[0]
+    from infinicore_infer_amd.engine.context import LayerCacheView
+    got = torch.empty(total, d, dtype=dtype)
+    pieces = [(0, cut), (cut, total - 3)] + [(i, i + 1) for i in range(total - 3, total)]
+    for a0, a1 in pieces:
+        ctx, _ = _context([(a0, a1 - a0)], 16, nkvh, dh, dtype)
+        cv = LayerCacheView(k=view.k, v=view.v, slots=view.slots[a0:a1].contiguous(),
+                            block_tables=view.block_tables)
+        got[a0:a1] = att.forward(h[a0:a1].to(DEV), ctx, cv).cpu()
+    assert _rel(got, want) < tol
+
+
+def test_embedding_and_head_parts():
+    from infinicore_infer_amd.parts import Runtime, build_part
+    from infinicore_infer_amd.config import PartSpec
+    rt = Runtime(torch.bfloat16, DEV)
+    emb = build_part("embedding", PartSpec("embedding", "e.", {"vocab_size": 77, "hidden_size": 40, "scale": 3.0}), rt)
+    head = build_part("head", PartSpec("lm_head", "h.", {"vocab_size": 77, "hidden_size": 40, "logit_scale": 0.5,
+                                                         "fallback_name": "e."}), rt)
+    norm = build_part("norm", PartSpec("rmsnorm", "n.", {"size": 40, "eps": 1e-5}), rt)
+    assert head.weight_specs()["h.weight"].fallback == "e.weight"
+    table = torch.randn(77, 40).to(torch.bfloat16)
+    nw = 1 + 0.1 * torch.randn(40)
+    emb.load_weights({"e.weight": table.to(DEV)})
+    head.load_weights({"h.weight": table.to(DEV)})
+    norm.load_weights({"n.weight": nw.to(DEV)})
+    toks = [5, 76, 0, 5]
+    x = torch.empty(4, 40, device=DEV)
+    emb.forward(torch.tensor(toks, dtype=torch.int32, device=DEV), x)
+    assert _rel(x, P.plain_embedding(table, toks, 3.0)) < 1e-6
+    ctx, _ = _context([(0, 4)], 16, 1, 16, torch.bfloat16)
+    rows = torch.tensor([3, 1], dtype=torch.int32, device=DEV)
+    logits = head.forward(x, rows, norm, ctx)
+    hn = P.round_bf16(P.plain_rmsnorm(x.cpu()[[3, 1]], nw, 1e-5) * 0.5)
+    assert logits.dtype == torch.float32 and _rel(logits, P.plain_linear(hn, table)) < 2e-3
+
+
+# ---------------------------------------------------------------------------
+# generation through the entry point and the scheduler
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("name", ["A", "B"])
+@pytest.mark.parametrize("dtype", [torch.float32, torch.bfloat16])
+def test_greedy_generation_through_the_entry_point(tmp_path_factory, name, dtype):
+    from infinicore_infer_amd.minicpm import MiniCPMForCausalLM
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), name, seed=7)
+    cfg = H.CONFIGS[name][0]
+    sd = H.load_state_dict(folder)
+    prompt = H.random_tokens(cfg["vocab_size"], 11, 8)
+    rnd = P.round_bf16 if dtype == torch.bfloat16 else None
+    want = P.plain_generate(dict(cfg, eos_token_id=[]), sd, prompt, 8, rnd=rnd)
+    model = MiniCPMForCausalLM(folder, DEV, 1, dtype=dtype, cache_tokens=256, page_size=16)
+    model.eos_token_id = []
+    out, _ = model.generate(prompt, 8)
+    assert model.last_output_tokens == want
+    # the same through the scheduler, three prompts at once, with so few pages that one is preempted
+    prompts = [prompt, prompt[:5], prompt[3:]]
+    wants = [P.plain_generate(dict(cfg, eos_token_id=[]), sd, p, 8, rnd=rnd) for p in prompts]
+    model2 = MiniCPMForCausalLM(folder, DEV, 1, dtype=dtype, cache_tokens=48, page_size=16)
+    model2.eos_token_id = []
+    assert model2.generate_batch(prompts, 8, max_batch_tokens=16, chunk_size=6) == wants
+    assert model2.engine.cache.free_pages(0) == 3
+    ppl = model.perplexity([prompt, prompt[2:]], batch_size=2)
+    logits = [P.plain_forward(cfg, sd, p[:-1], rnd=rnd) for p in (prompt, prompt[2:])]
+    nll = sum(-float(torch.log_softmax(l, -1)[torch.arange(len(p) - 1), torch.tensor(p[1:])].sum())
+              for l, p in zip(logits, (prompt, prompt[2:])))
+    assert ppl == pytest.approx(math.exp(nll / (len(prompt) - 1 + len(prompt) - 3)), rel=2e-2 if rnd else 1e-4)
+
+
+def test_temperature_sampling_is_reproducible(tmp_path_factory):
+    from infinicore_infer_amd.minicpm import MiniCPMForCausalLM
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "B", seed=7)
+    model = MiniCPMForCausalLM(folder, DEV, 1, dtype=torch.float32, cache_tokens=256, page_size=16)
+    model.eos_token_id = []
+    prompts = [H.random_tokens(509, 9, 1), H.random_tokens(509, 4, 2)]
+    a = model.generate_batch(prompts, 12, topp_=0.9, topk_=40, temperature_=1.5, seed=3)
+    b = model.generate_batch(prompts, 12, topp_=0.9, topk_=40, temperature_=1.5, seed=3)
+    c = model.generate_batch(prompts, 12, topp_=0.9, topk_=40, temperature_=1.5, seed=4)
+    assert a == b and a != c
+
+
+# ---------------------------------------------------------------------------
+# a toy architecture, defined and registered here
+# ---------------------------------------------------------------------------
+def _register_toy():
+    from infinicore_infer_amd.config import ExecEntry, LayerSpec, ModelSpec, PartSpec, register_architecture
+    from infinicore_infer_amd.parts import CacheNeed, Mixer, register_part
+    from infinicore_infer_amd.weights import WeightSpec
+
+    @register_part("mixer", "toy_running_mean")
+    class RunningMean(Mixer):
+        """y_t = gain * mean(h_0..h_t): needs a running sum and a count per request."""
+
+        def __init__(self, name, runtime, hidden_size):
+            super().__init__(name, runtime)
+            self.d = hidden_size
+            self.gain = None
+
+        def cache_need(self):
+            return CacheNeed("state", state_shape=(self.d + 1,), state_dtype=torch.float32)
+
+        def weight_specs(self):
+            return {self.name + "gain": WeightSpec((self.d,), "vector")}
+
+        def load_weights(self, tensors):
+            self.gain = tensors[self.name + "gain"]
+
+        def forward(self, h, ctx, cache):
+            y = ctx.ws.buffer("toy_out", tuple(h.shape), self.runtime.dtype)
+            for r in range(ctx.R):
+                a, b = ctx.req_start[r], ctx.req_start[r + 1]
+                st = cache.state[ctx.host_state_slots[r]]
+                cs = torch.cumsum(h[a:b].float(), 0) + st[:-1]
+                n = st[-1] + torch.arange(1, b - a + 1, device=h.device)
+                y[a:b] = (cs / n[:, None] * self.gain).to(y.dtype)
+                st[:-1] = cs[-1]
+                st[-1] = n[-1]
+            return y
+
+    class ToyConfig:
+        def __init__(self, cfg):
+            self.cfg = cfg
+
+        @classmethod
+        def from_dict(cls, cfg, **kw):
+            return cls(cfg)
+
+        def model_spec(self):
+            c = self.cfg
+            d, nh, nkvh, dh = c["hidden"], c["heads"], c["kv_heads"], c["head_dim"]
+            rot = PartSpec("rotary", "", {"head_dim": dh, "theta": 1000.0, "max_positions": c["max_pos"]})
+
+            def norm(p):
+                return PartSpec("rmsnorm", p, {"size": d, "eps": 1e-5})
+
+            def ffn(p):
+                return PartSpec("swiglu", p, {"hidden_size": d, "intermediate_size": c["inter"]})
+
+            def attn(p, **kw):
+                return PartSpec("attention", p, dict({"hidden_size": d, "num_heads": nh, "num_kv_heads": nkvh,
+                                                      "head_dim": dh, "softmax_scale": dh ** -0.5,
+                                                      "position_encoding": rot}, **kw))
+            block = lambda p: PartSpec("prenorm_residual", p, {"residual_scale": 0.8})
+            layers = [
+                LayerSpec(block("l0."), attn("l0.att.", window=c["window"]), norm("l0.n1."), ffn("l0.ffn."), norm("l0.n2.")),
+                LayerSpec(block("l1."), PartSpec("toy_running_mean", "l1.mix.", {"hidden_size": d}), norm("l1.n1."),
+                          ffn("l1.ffn."), norm("l1.n2.")),
+                LayerSpec(block("l2."), attn("l2.att.", window=c["window"], shared_kv=True), norm("l2.n1."),
+                          ffn("l2.ffn."), norm("l2.n2.")),
+                LayerSpec(block("l3."), attn("l3.att."), norm("l3.n1."), ffn("l3.ffn."), norm("l3.n2.")),
+            ]
+            schedule = [ExecEntry(0, 0, True), ExecEntry(1, 1, True), ExecEntry(2, 0, False),
+                        ExecEntry(3, 2, True), ExecEntry(1, 3, True)]       # layer 1 runs twice, each run with its own state
+            return ModelSpec("toy", c["vocab"], d, c["max_pos"],
+                             PartSpec("embedding", "emb.", {"vocab_size": c["vocab"], "hidden_size": d, "scale": 2.0}),
+                             layers, schedule, norm("final."),
+                             PartSpec("lm_head", "head.", {"vocab_size": c["vocab"], "hidden_size": d, "logit_scale": 1.0,
+                                                           "fallback_name": "emb."}))
+
+    register_architecture(["toy-test-arch"], ToyConfig)
+
+
+def _toy_plain(model, cfg, tokens):
+    """The toy model in plain float64, whole sequence."""
+    T = len(tokens)
+    d, nh, nkvh, dh, win = cfg["hidden"], cfg["heads"], cfg["kv_heads"], cfg["head_dim"], cfg["window"]
+    half = dh // 2
+    cpu = lambda t: t.detach().cpu().double()
+    sin, cos = P.plain_rope_tables(dh, 1000.0, T)
+
+    def rope(x):
+        s, c = sin[:T, None, :], cos[:T, None, :]
+        return torch.cat([x[..., :half] * c - x[..., half:] * s, x[..., :half] * s + x[..., half:] * c], -1)
+
+    x = P.plain_embedding(cpu(model.embedding.table), tokens, 2.0)
+    kv = {}
+    for e in model.schedule:
+        blk = model.layers[e.layer]
+        h = P.plain_rmsnorm(x, cpu(blk.mixer_norm.weight), 1e-5)
+        m = blk.mixer
+        if hasattr(m, "gain"):
+            y = torch.cumsum(h, 0) / torch.arange(1, T + 1)[:, None] * cpu(m.gain)
+        else:
+            qkv = P.plain_linear(h, cpu(m.w_qkv))
+            q = rope(qkv[:, :nh * dh].reshape(T, nh, dh))
+            if e.writes_cache:
+                k = rope(qkv[:, nh * dh:(nh + nkvh) * dh].reshape(T, nkvh, dh))
+                v = qkv[:, (nh + nkvh) * dh:].reshape(T, nkvh, dh)
+                kv[e.cache] = (k, v)
+            k, v = kv[e.cache]
+            a = P.plain_attention(q, k, v, dh ** -0.5, 0, m.window or None).reshape(T, nh * dh)
+            y = P.plain_linear(a, cpu(m.w_o))
+        x = x + 0.8 * y
+        h = P.plain_rmsnorm(x, cpu(blk.feed_forward_norm.weight), 1e-5)
+        gu = P.plain_linear(h, cpu(blk.feed_forward.w_gate_up))
+        di = gu.shape[1] // 2
+        x = x + 0.8 * P.plain_linear(P.plain_swiglu(gu[:, :di], gu[:, di:]), cpu(blk.feed_forward.w_down))
+    return P.plain_linear(P.plain_rmsnorm(x, cpu(model.final_norm.weight), 1e-5), cpu(model.head.weight))
+
+
+def test_toy_architecture_with_a_stateful_mixer(tmp_path_factory):
+    from infinicore_infer_amd.config import config_from_dict
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.parts import Runtime, build_model
+    from infinicore_infer_amd.weights import init_random_weights
+    _register_toy()
+    cfg = {"model_type": "toy-test-arch", "vocab": 97, "hidden": 48, "heads": 4, "kv_heads": 2, "head_dim": 16,
+           "inter": 80, "window": 24, "max_pos": 256}
+    model = build_model(config_from_dict(cfg).model_spec(), Runtime(torch.float32, DEV))
+    init_random_weights(model, seed=11, std=0.15, norm_std=0.1, tie=True)
+    needs = model.cache_needs()
+    assert [n.kind for n in needs] == ["kv", "state", "kv", "state"]
+    assert needs[0].window == 24 and needs[2].window is None
+    requests = {"t%d" % i: H.random_tokens(97, n, 40 + i) for i, n in enumerate([70, 33, 120, 9])}
+    ref = {rid: _toy_plain(model, cfg, toks) for rid, toks in requests.items()}
+    for maker in (H.trace_whole, H.trace_chunks, H.trace_mixed):
+        steps, max_tokens = maker(requests)
+        eng = Engine(model, max_tokens=max_tokens, page_size=16, max_requests=4)
+        assert len(eng.groups) == 2 and {g.kind for g in eng.groups} == {"full", "window"}
+        got = H.run_trace(eng, steps)
+        H.compare(got, ref, 1e-4, "toy %s" % maker.__name__)
+        eng.cache.check_invariants()
+        assert all(eng.cache.free_pages(g) == eng.num_pages for g in range(2))
+    # the window group really gives pages back while a long request runs
+    eng = Engine(model, max_tokens=128, page_size=16, max_requests=2)
+    from infinicore_infer_amd.engine import StepEntry
+    eng.step([StepEntry("w", requests["t2"][:100], [])])
+    wg = [i for i, g in enumerate(eng.groups) if g.kind == "window"][0]
+    assert eng.cache.free_pages(wg) > eng.cache.free_pages(1 - wg)

@@ -1,0 +1,183 @@
+"""The scheduler's decisions with a stand-in engine (real cache manager, no GPU). (CPU)"""
+import hashlib
+
+import pytest
+
+from infinicore_infer_amd.cache import CacheManager, GroupSpec, OutOfPages
+from infinicore_infer_amd.engine.scheduler import Scheduler
+from infinicore_infer_amd.engine.tasks import InferTask
+
+VOCAB = 50
+
+
+def _next_token(history):
+    h = hashlib.sha256(",".join(map(str, history)).encode()).digest()
+    return h[0] % VOCAB
+
+
+class FakeEngine:
+    """Keeps each request's token history and 'predicts' a token that is a pure function of it,
+    so a recomputed request must reproduce its continuation.  Checks what the scheduler feeds."""
+
+    def __init__(self, num_pages, page_size=16, max_requests=4, max_positions=None):
+        self.cache = CacheManager([GroupSpec("full", 1, 16, None, (0,))], num_pages, page_size, max_requests,
+                                  max_positions)
+        self.history = {}
+        self.steps = []
+
+    def add_request(self, rid):
+        self.cache.admit(rid)
+        self.history[rid] = []
+
+    def free(self, rid):
+        if self.cache.has_request(rid):
+            self.cache.release(rid)
+            del self.history[rid]
+
+    def step(self, entries):
+        assert len({e.req_id for e in entries}) == len(entries)
+        rows = []
+        for e in entries:
+            start = self.cache.append(e.req_id, len(e.tokens))       # raises OutOfPages if the plan was wrong
+            assert start == len(self.history[e.req_id])
+            self.history[e.req_id].extend(e.tokens)
+            for w in e.want:
+                rows.append(_next_token(self.history[e.req_id][:start + w + 1]))
+        self.steps.append([(e.req_id, len(e.tokens)) for e in entries])
+        self.cache.check_invariants()
+        return rows
+
+    def sample(self, logits, temperature=None, top_k=None, top_p=None, uniform=None):
+        return list(logits)
+
+
+def _expected(prompt, n, end=()):
+    toks, out = list(prompt), []
+    for _ in range(n):
+        t = _next_token(toks)
+        out.append(t)
+        toks.append(t)
+        if t in end:
+            break
+    return out
+
+
+def _task(i, prompt, new, end=()):
+    return InferTask(i, prompt, max_tokens=10 ** 6, end_tokens=list(end), max_new_tokens=new)
+
+
+def test_prompts_are_cut_under_the_token_budget_and_decodes_come_first():
+    eng = FakeEngine(num_pages=64)
+    s = Scheduler(eng, max_batch_tokens=40, chunk_size=32)
+    s.add(_task("a", list(range(70)), 3))
+    s.add(_task("b", list(range(10)), 3))
+    s.step()
+    assert eng.steps[-1] == [("a", 32), ("b", 8)]         # a's portion, then what the budget leaves for b
+    s.step()
+    assert eng.steps[-1] == [("a", 32), ("b", 2)]
+    s.step()
+    assert eng.steps[-1] == [("b", 1), ("a", 6)]          # b decodes first, then a's last portion
+    while s.has_unfinished():
+        s.step()
+        assert sum(n for _, n in eng.steps[-1]) <= 40
+        ones = [n for _, n in eng.steps[-1]]
+        assert ones == sorted(ones)                       # single decode tokens are listed before portions
+    done = {t.id: t for t in s.finished}
+    assert done["a"].generated == _expected(range(70), 3) and done["b"].generated == _expected(range(10), 3)
+    assert done["a"].finish_reason == "length"
+    assert eng.cache.free_pages() == 64 and not eng.cache.requests
+
+
+def test_budget_is_shared_first_come_first_served():
+    eng = FakeEngine(num_pages=64)
+    s = Scheduler(eng, max_batch_tokens=48, chunk_size=32)
+    for i, n in enumerate([20, 20, 20]):
+        s.add(_task(i, list(range(n)), 2))
+    s.step()
+    assert eng.steps[-1] == [(0, 20), (1, 20), (2, 8)]
+    s.step()
+    assert eng.steps[-1] == [(0, 1), (1, 1), (2, 12)]
+
+
+def test_end_tokens_and_position_limit():
+    eng = FakeEngine(num_pages=16)
+    s = Scheduler(eng)
+    prompt = [3, 1, 4, 1, 5]
+    full = _expected(prompt, 30)
+    stop = full[4]
+    t1 = InferTask("s", prompt, max_tokens=10 ** 6, end_tokens=[stop], max_new_tokens=30)
+    t2 = InferTask("l", prompt, max_tokens=9, end_tokens=[], max_new_tokens=None)
+    s.add(t1)
+    s.add(t2)
+    s.run()
+    assert t1.finish_reason == "stop" and t1.generated == full[:full.index(stop) + 1]
+    assert t2.finish_reason == "length" and t2.pos == 9 and t2.generated == full[:5]   # scripts/infer_task.py:33
+
+
+def test_running_out_of_pages_preempts_the_youngest_and_recomputes_the_same_tokens():
+    eng = FakeEngine(num_pages=6, page_size=16, max_requests=4)           # 96 token slots
+    s = Scheduler(eng, max_batch_tokens=64, chunk_size=32)
+    prompts = {"a": list(range(30)), "b": list(range(5, 35)), "c": list(range(9, 39))}
+    for k, p in prompts.items():
+        s.add(_task(k, p, 40))
+    done = s.run()
+    assert s.n_preempted > 0
+    for t in done:
+        assert t.generated == _expected(prompts[t.id], 40), t.id
+        assert t.finish_reason == "length"
+    assert eng.cache.free_pages() == 6 and eng.cache.slots.n_free == 4
+    # the oldest request was never the victim: it was computed exactly once
+    fed_a = sum(n for step in eng.steps for rid, n in step if rid == "a")
+    assert fed_a == 30 + 39
+
+
+def test_a_request_too_large_for_the_cache_ends_with_length():
+    eng = FakeEngine(num_pages=2, page_size=16)
+    s = Scheduler(eng, max_batch_tokens=64, chunk_size=64)
+    big = _task("big", list(range(40)), 5)
+    ok = _task("ok", list(range(10)), 30)
+    s.add(big)
+    s.add(ok)
+    s.run()
+    assert big.finish_reason == "length" and big.generated == []
+    assert ok.finish_reason == "length" and ok.generated == _expected(range(10), 30)[:len(ok.generated)]
+    assert len(ok.generated) >= 22                      # it ran until the two pages were full
+    assert eng.cache.free_pages() == 2
+
+
+def test_admission_waits_for_slots_and_is_first_come_first_served():
+    eng = FakeEngine(num_pages=64, max_requests=2)
+    s = Scheduler(eng, max_batch_tokens=256, chunk_size=64)
+    for i in range(5):
+        s.add(_task(i, list(range(i, i + 6)), 4))
+    order = []
+    while s.has_unfinished():
+        s.step()
+        assert len(eng.cache.requests) <= 2
+        for rid, _ in eng.steps[-1]:
+            if rid not in order:
+                order.append(rid)
+    assert order == [0, 1, 2, 3, 4]
+    assert all(t.generated == _expected(range(t.id, t.id + 6), 4) for t in s.finished)
+
+
+def test_abort_frees_everything():
+    eng = FakeEngine(num_pages=8)
+    s = Scheduler(eng)
+    s.add(_task("x", list(range(20)), 50))
+    s.add(_task("y", list(range(20)), 50))
+    s.step()
+    s.abort("x")
+    s.abort("y")
+    assert not s.has_unfinished() and eng.cache.free_pages() == 8
+    assert {t.finish_reason for t in s.finished} == {"cancel"}
+
+
+def test_sampling_draws_do_not_depend_on_preemption():
+    from infinicore_infer_amd.sampling import SamplingParams, uniform_draw
+    assert uniform_draw(1, "r", 5) == uniform_draw(1, "r", 5) != uniform_draw(1, "r", 6)
+    assert 0.0 <= uniform_draw(2, 7, 0) < 1.0
+    assert SamplingParams().greedy and SamplingParams(temperature=0.0, topk=50).greedy
+    assert not SamplingParams(temperature=0.8, topk=50).greedy
+    with pytest.raises(ValueError):
+        SamplingParams(topp=1.5)
