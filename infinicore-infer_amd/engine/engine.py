@@ -32,6 +32,16 @@ def _align4(n: int) -> int:
     return (n + 3) & ~3
 
 
+def _context_bucket(n_keys: int) -> int:
+    """Key counts are rounded up to a power of two (at least 256) before the key split of
+    single-token rows is chosen, so eager and recorded steps split alike and a recorded
+    graph serves a whole range of lengths."""
+    b = 256
+    while b < n_keys:
+        b *= 2
+    return b
+
+
 class _PinnedRing:
     """A few pinned host buffers used in turn, each guarded by an event, so a
     buffer is not rewritten while its copy to the device may still run."""
@@ -61,7 +71,7 @@ class _PinnedRing:
 
 class Engine:
     def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 64,
-                 num_pages: Optional[int] = None):
+                 num_pages: Optional[int] = None, use_graphs: bool = True, graph_max_batch: int = 64):
         """``max_tokens``: the most tokens live requests hold at any time, each
         request's count rounded up to whole pages; every group's pool is sized for it."""
         self.model = model
@@ -103,6 +113,11 @@ class Engine:
         self._tile_rows = ops.attention_prefill_tile_rows()
         self.cu_count = torch.cuda.get_device_properties(self.device).multi_processor_count
         self.steps_run = 0
+        # decode steps (one token per request, its logits wanted) replay a captured HIP graph
+        self.use_graphs = bool(use_graphs) and all(p.graph_safe for p in model.all_parts())
+        self.graph_max_batch = int(graph_max_batch)
+        self._graphs: Dict[tuple, "_DecodeGraph"] = {}
+        self.graph_replays = 0
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
@@ -175,8 +190,12 @@ class Engine:
             self.add_request(rid)
         starts = [self.cache.append(e.req_id, len(e.tokens)) for e in entries]
 
-        ctx = self._build_context(entries, starts)
-        logits = self.model.forward(ctx)
+        if (self.use_graphs and len(entries) <= self.graph_max_batch
+                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
+            logits = self._graph_step(entries, starts)
+        else:
+            ctx = self._build_context(entries, starts)
+            logits = self.model.forward(ctx)
         for e in entries:
             self.cache.trim(e.req_id)
         self.steps_run += 1
@@ -265,7 +284,7 @@ class Engine:
         ctx.req_ids = [e.req_id for e in entries]
         ctx.host_state_slots = state_slots
         ctx.max_position = max(positions)
-        ctx.max_context = max_ctx
+        ctx.max_context = _context_bucket(max_ctx) if max_ctx else 0
         ctx.cu_count = self.cu_count
         for slot in range(self.model.spec.num_cache_slots()):
             if slot in self._slot_group:
@@ -276,6 +295,36 @@ class Engine:
             else:
                 ctx._views[slot] = LayerCacheView(state=self.storage.state.get(slot))
         return ctx
+
+    # ---- decode steps as captured graphs ------------------------------------------------------------
+    def _graph_step(self, entries, starts):
+        """A step of single tokens, one per request, all logits wanted.  The kernels of
+        such a step differ from step to step only in the integers they read (tokens,
+        positions, slots, block tables), so the launch sequence is captured once per
+        (batch size, key split) into a HIP graph with those integers in a fixed device
+        buffer, and replayed after one copy into that buffer."""
+        R = len(entries)
+        ps = self.page_size
+        bucket = _context_bucket(max(starts) + 1)
+        key = (R, bucket)
+        g = self._graphs.get(key)
+        if g is None:
+            g = _DecodeGraph(self, R, bucket)
+            self._graphs[key] = g
+        host = self._ring.get(g.total)
+        flat = g.fill(self, entries, starts)
+        host[:g.total] = torch.tensor(flat, dtype=torch.int32)
+        g.meta[:g.total].copy_(host[:g.total], non_blocking=True)
+        self._ring.mark()
+        g.ctx.max_position = max(starts)
+        g.ctx.req_pos = list(starts)
+        g.ctx.req_ids = [e.req_id for e in entries]
+        g.ctx.host_state_slots = flat[g.off["state_slots"]:g.off["state_slots"] + R]
+        if g.graph is None:
+            g.capture(self)
+        g.graph.replay()
+        self.graph_replays += 1
+        return g.logits
 
     # ---- sampling --------------------------------------------------------------------------------------
     def sample(self, logits, temperature=None, top_k=None, top_p=None, uniform=None) -> List[int]:
@@ -290,3 +339,85 @@ class Engine:
             k = torch.tensor(list(top_k), dtype=torch.int32).to(self.device)
             ops.sample(logits, out, f[0].contiguous(), k, f[1].contiguous(), f[2].contiguous())
         return out.cpu().tolist()
+
+
+class _DecodeGraph:
+    """Fixed layout of a decode step's integers for R requests, the step context
+    built on views of it, and the captured graph."""
+
+    def __init__(self, engine: "Engine", R: int, ctx_bucket: int):
+        self.R = R
+        ng = len(engine.groups)
+        self.maxb = (engine.model.spec.max_positions + engine.page_size - 1) // engine.page_size
+        names = ["tokens", "positions", "token_req", "state_slots", "want_rows"]
+        sizes = {n: R for n in names}
+        for g in range(ng):
+            names += ["slots%d" % g, "tables%d" % g]
+            sizes["slots%d" % g] = R
+            sizes["tables%d" % g] = R * self.maxb
+        self.off, total = {}, 0
+        for n in names:
+            self.off[n] = total
+            total += _align4(sizes[n])
+        self.total = total
+        self.sizes = sizes
+        self.meta = torch.zeros(total, dtype=torch.int32, device=engine.device)
+        self.graph = None
+        self.logits = None
+
+        def view(n):
+            return self.meta[self.off[n]:self.off[n] + sizes[n]]
+
+        ctx = StepContext()
+        # a workspace of its own: the recorded launches hold its addresses, so it must never be regrown
+        ctx.T, ctx.R, ctx.page_size, ctx.ws = R, R, engine.page_size, Workspace(engine.device)
+        ctx.tokens, ctx.positions, ctx.token_req = view("tokens"), view("positions"), view("token_req")
+        ctx.state_slots = view("state_slots")
+        ctx.want_rows, ctx.n_want = view("want_rows"), R
+        ctx.decode_rows, ctx.n_decode_rows, ctx.decode_rows_identity = None, R, True
+        ctx.prefill_tiles, ctx.n_prefill_tiles = None, 0
+        ctx.req_start = list(range(R + 1))
+        ctx.req_len = [1] * R
+        ctx.max_context = ctx_bucket
+        ctx.cu_count = engine.cu_count
+        for slot in range(engine.model.spec.num_cache_slots()):
+            if slot in engine._slot_group:
+                g = engine._slot_group[slot]
+                k, v = engine.storage.kv(slot)
+                ctx._views[slot] = LayerCacheView(k=k, v=v, slots=view("slots%d" % g),
+                                                  block_tables=view("tables%d" % g).view(R, self.maxb))
+            else:
+                ctx._views[slot] = LayerCacheView(state=engine.storage.state.get(slot))
+        self.ctx = ctx
+
+    def fill(self, engine, entries, starts):
+        R, ps = self.R, engine.page_size
+        flat = [0] * self.total
+        o = self.off
+        for r, (e, p0) in enumerate(zip(entries, starts)):
+            flat[o["tokens"] + r] = int(e.tokens[0])
+            flat[o["positions"] + r] = p0
+            flat[o["token_req"] + r] = r
+            flat[o["state_slots"] + r] = engine.cache.state_slot(e.req_id)
+            flat[o["want_rows"] + r] = r
+            for g in range(len(engine.groups)):
+                table = engine.cache.block_table(e.req_id, g)
+                flat[o["slots%d" % g] + r] = table[p0 // ps] * ps + p0 % ps
+                base = o["tables%d" % g] + r * self.maxb
+                for j, p in enumerate(table):
+                    flat[base + j] = p if p > 0 else 0
+        return flat
+
+    def capture(self, engine):
+        """Run the step once eagerly (every buffer then exists and the result is
+        already right), then record the same launches."""
+        engine.model.forward(self.ctx)
+        torch.cuda.synchronize()
+        graph = torch.cuda.CUDAGraph()
+        stream = torch.cuda.Stream()
+        stream.wait_stream(torch.cuda.current_stream())
+        with torch.cuda.stream(stream):
+            with torch.cuda.graph(graph, stream=stream):
+                self.logits = engine.model.forward(self.ctx)
+        torch.cuda.current_stream().wait_stream(stream)
+        self.graph = graph

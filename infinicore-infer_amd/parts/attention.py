@@ -20,6 +20,8 @@ from .linear import linear
 
 @register_part("mixer", "attention")
 class Attention(Mixer):
+    graph_safe = True
+
     def __init__(self, name, runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  softmax_scale: float, position_encoding, window=None, shared_kv: bool = False):
         super().__init__(name, runtime)

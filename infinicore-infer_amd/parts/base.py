@@ -75,6 +75,10 @@ def build_part(category: str, spec: PartSpec, runtime: Runtime, memo: Optional[d
 class Part:
     """Base of all parts."""
     category = ""
+    # True when forward() launches the same kernels with the same arguments for every step of
+    # a given batch shape and reads the step's integers only from device arrays (never from the
+    # context's host lists): such a step can be recorded once and replayed.
+    graph_safe = False
 
     def __init__(self, name: str, runtime: Runtime):
         self.name = name

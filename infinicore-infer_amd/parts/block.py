@@ -12,6 +12,8 @@ from .base import Block, register_part
 
 @register_part("block", "prenorm_residual")
 class PreNormResidualBlock(Block):
+    graph_safe = True
+
     def __init__(self, name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm,
                  residual_scale: float = 1.0):
         super().__init__(name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm)

@@ -18,6 +18,8 @@ from .linear import linear
 
 @register_part("embedding", "embedding")
 class Embedding(Part):
+    graph_safe = True
+
     category = "embedding"
 
     def __init__(self, name, runtime, vocab_size: int, hidden_size: int, scale: float = 1.0,
@@ -40,6 +42,8 @@ class Embedding(Part):
 
 @register_part("head", "lm_head")
 class LMHead(Part):
+    graph_safe = True
+
     category = "head"
 
     def __init__(self, name, runtime, vocab_size: int, hidden_size: int, logit_scale: float = 1.0,

@@ -9,6 +9,8 @@ from .base import Norm, register_part
 
 @register_part("norm", "rmsnorm")
 class RMSNorm(Norm):
+    graph_safe = True
+
     def __init__(self, name, runtime, size: int, eps: float):
         super().__init__(name, runtime)
         self.size = size

@@ -44,6 +44,8 @@ _TABLES = {}
 
 @register_part("position_encoding", "rotary")
 class Rotary(PositionEncoding):
+    graph_safe = True
+
     def __init__(self, name, runtime, head_dim: int, theta: float, max_positions: int, scaling=None,
                  rot_dim=None):
         super().__init__(name, runtime)
@@ -69,6 +71,8 @@ class Rotary(PositionEncoding):
 
 @register_part("position_encoding", "none")
 class NoPositionEncoding(PositionEncoding):
+    graph_safe = True
+
     """No rotation: only the cache write."""
 
     def __init__(self, name, runtime, **_):

@@ -15,6 +15,8 @@ from .linear import linear
 
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
+    graph_safe = True
+
     def __init__(self, name, runtime, hidden_size: int, intermediate_size: int):
         super().__init__(name, runtime)
         self.hidden_size = hidden_size

@@ -133,3 +133,63 @@ def test_bad_tokens_are_refused(tmp_path_factory):
     with pytest.raises(ValueError):
         engine.step([StepEntry("z", [1, 2], [2])])
     assert not engine.has_request("z")
+
+
+@pytest.mark.parametrize("dname,dtype,tol", DTYPES)
+def test_recorded_decode_steps_equal_eager_ones(tmp_path_factory, dname, dtype, tol):
+    """Decode steps replay a recorded graph.  Every replay is checked against the same step run
+    eagerly by a second engine, with eager work (prompt portions, synchronising copies) between
+    the replays, for two batch sizes and across a change of the key-split bucket."""
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "C")
+    a = Engine.from_dir(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4, use_graphs=True)
+    b = Engine.from_dir(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4, use_graphs=False)
+    prompts = {"p": H.random_tokens(331, 250, 1), "q": H.random_tokens(331, 40, 2), "r": H.random_tokens(331, 90, 3)}
+    for eng in (a, b):
+        eng.step([StepEntry("p", prompts["p"], []), StepEntry("q", prompts["q"], [])])
+    toks = H.random_tokens(331, 40, 9)
+    for i in range(12):                      # two requests; "p" crosses 256 keys: a new bucket, a new graph
+        la = a.step([StepEntry("p", [toks[i]], [0]), StepEntry("q", [toks[i + 1]], [0])]).clone()
+        lb = b.step([StepEntry("p", [toks[i]], [0]), StepEntry("q", [toks[i + 1]], [0])]).clone()
+        assert torch.equal(la, lb), "replay %d differs from the eager step" % i
+        if i == 5:                           # eager work in between: a third request's prompt
+            for eng in (a, b):
+                eng.step([StepEntry("r", prompts["r"], [])])
+    for i in range(6):                       # three requests
+        ents = [StepEntry(k, [toks[20 + i + j]], [0]) for j, k in enumerate("pqr")]
+        assert torch.equal(a.step(ents).clone(), b.step(ents).clone())
+    assert a.graph_replays == 18 and b.graph_replays == 0 and len(a._graphs) >= 3
+
+
+def test_trace_run_program(tmp_path):
+    """bin/trace_run as a program: files, 'done' lines, exit status, and the logits themselves."""
+    import json, os, subprocess, sys
+    import numpy as np
+    folder = H.make_model_dir(tmp_path, "A", seed=2)
+    cfg = H.CONFIGS["A"][0]
+    requests = {"a": H.random_tokens(256, 50, 1), "b": H.random_tokens(256, 21, 2)}
+    steps, max_tokens = H.trace_mixed(requests, sizes=(9, 2, 5))
+    steps[1]["entries"][0]["want"] = []                       # a step entry that wants nothing
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    for dname, tol in (("float32", H.FP32_TOL), ("bfloat16", H.BF16_TOL)):
+        out = tmp_path / ("out_" + dname)
+        p = subprocess.run([os.path.join(root, "bin", "trace_run"), "--model", folder, "--dtype", dname,
+                            "--out", str(out), "--max-tokens", str(max_tokens)],
+                           input="".join(json.dumps(s) + "\n" for s in steps), capture_output=True, text=True,
+                           timeout=300)
+        assert p.returncode == 0, p.stderr[-2000:]
+        assert p.stdout.split("\n")[:-1] == ["done %d" % s["step"] for s in steps]
+        ref = H.plain_logits(cfg, H.load_state_dict(folder), requests, dname == "bfloat16")
+        cursor, got = {}, {}
+        for s in steps:
+            n_want = sum(len(e["want"]) for e in s["entries"])
+            path = out / ("%d.f32" % s["step"])
+            assert path.exists() == (n_want > 0)
+            rows = np.fromfile(path, dtype="<f4").reshape(n_want, 256) if n_want else None
+            i = 0
+            for e in s["entries"]:
+                for w in e["want"]:
+                    got[(e["id"], cursor.get(e["id"], 0) + w)] = torch.from_numpy(rows[i].copy())
+                    i += 1
+                cursor[e["id"]] = cursor.get(e["id"], 0) + len(e["tokens"])
+        H.compare(got, ref, tol, "trace_run " + dname)
