@@ -187,27 +187,29 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
     }
 }
 
+// Grid (tokens * heads), one wave.  Lane s holds split s (at most 64 splits): the
+// weights exp(m_s - max) come from one wave reduction; every lane then sums its
+// output dims over the splits with independent loads.
 template <typename T>
-__global__ void attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
-                                          const int* __restrict__ tok_list, T* __restrict__ out,
-                                          int out_stride, int nh, int dh, int nsplit) {
-    const int n = blockIdx.x / nh, h = blockIdx.x % nh;
+__global__ void __launch_bounds__(64)
+attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
+                          const int* __restrict__ tok_list, T* __restrict__ out,
+                          int out_stride, int nh, int dh, int nsplit) {
+    __shared__ float wgt[64];
+    const int n = blockIdx.x / nh, h = blockIdx.x % nh, lane = threadIdx.x;
     const int t = tok_list ? tok_list[n] : n;
     const size_t base = ((size_t)n * nh + h) * nsplit;
-    float mm = -INFINITY;
-    for (int s = 0; s < nsplit; ++s) mm = fmaxf(mm, part_ml[(base + s) * 2]);
-    float ll = 0.f;
-    for (int s = 0; s < nsplit; ++s) {
-        const float ms = part_ml[(base + s) * 2];
-        if (ms != -INFINITY) ll += part_ml[(base + s) * 2 + 1] * expf(ms - mm);
-    }
-    const float inv = 1.0f / ll;
-    for (int d = threadIdx.x; d < dh; d += blockDim.x) {
+    float ms = -INFINITY, ls = 0.f;
+    if (lane < nsplit) { ms = part_ml[(base + lane) * 2]; ls = part_ml[(base + lane) * 2 + 1]; }
+    const float mm = wave_max(ms);
+    const float w = (ms == -INFINITY) ? 0.f : expf(ms - mm);
+    const float inv = 1.0f / wave_sum(ls * w);
+    wgt[lane] = w;
+    __syncthreads();
+    for (int d = lane; d < dh; d += 64) {
         float a = 0.f;
-        for (int s = 0; s < nsplit; ++s) {
-            const float ms = part_ml[(base + s) * 2];
-            if (ms != -INFINITY) a += part_acc[(base + s) * dh + d] * expf(ms - mm);
-        }
+#pragma unroll 4
+        for (int s = 0; s < nsplit; ++s) a += part_acc[(base + s) * dh + d] * wgt[s];
         out[(size_t)t * out_stride + (size_t)h * dh + d] = from_f32<T>(a * inv);
     }
 }
@@ -248,7 +250,7 @@ IC_EXPORT int ic_attn_decode(const void* q, int q_stride, void* out, int out_str
                              int nkvh, int dh, int page_size, float scale, int window, int nsplit,
                              hipStream_t stream) {
     if (n_tok <= 0) return IC_OK;
-    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || nsplit <= 0) return IC_ERR_ARG;
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || nsplit <= 0 || nsplit > 64) return IC_ERR_ARG;
     if (nkvh > 65535 || n_tok > 65535) return IC_ERR_ARG;
     if (q_stride % 8 || ((uintptr_t)q & 15) || ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15)) return IC_ERR_ARG;
 #define IC_DECODE_CASE(TT, DD)                                                                          \

@@ -30,6 +30,96 @@ IC_EXPORT int ic_embed(const int* tokens, const void* table, int table_dtype, fl
     return ic_launch_status();
 }
 
+// ---- four elements at a time ----------------------------------------------------
+__device__ __forceinline__ void load4(const float* p, float* o) {
+    const float4 v = *reinterpret_cast<const float4*>(p);
+    o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+}
+__device__ __forceinline__ void load4(const bf16* p, float* o) {
+    const uint2 v = *reinterpret_cast<const uint2*>(p);
+    o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
+    o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
+}
+__device__ __forceinline__ void store4(float* p, const float* o) {
+    *reinterpret_cast<float4*>(p) = make_float4(o[0], o[1], o[2], o[3]);
+}
+__device__ __forceinline__ void store4(bf16* p, const float* o) {
+    uint2 v;
+    v.x = (uint32_t)f32_to_bf16_bits(o[0]) | ((uint32_t)f32_to_bf16_bits(o[1]) << 16);
+    v.y = (uint32_t)f32_to_bf16_bits(o[2]) | ((uint32_t)f32_to_bf16_bits(o[3]) << 16);
+    *reinterpret_cast<uint2*>(p) = v;
+}
+
+// One pass: a row lives in registers between the sum of squares and the scaling
+// (d % 4 == 0, d <= 4 * VPT * blockDim).  ADD: x += alpha * y first, x written back.
+template <typename TY, typename TO, int VPT, bool ADD>
+__global__ void norm_row_kernel(float* __restrict__ x, const int* __restrict__ rows, const TY* __restrict__ y,
+                                float alpha, const float* __restrict__ w, TO* __restrict__ out, int d,
+                                float eps, float out_scale) {
+    __shared__ float red[16];
+    const int r = blockIdx.x;
+    float* xr = x + (size_t)(rows ? rows[r] : r) * d;
+    float v[VPT][4];
+    float ss = 0.f;
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = 4 * (threadIdx.x + i * blockDim.x);
+        if (c < d) {
+            load4(xr + c, v[i]);
+            if (ADD) {
+                float yv[4];
+                load4(y + (size_t)r * d + c, yv);
+#pragma unroll
+                for (int e = 0; e < 4; ++e) v[i][e] += alpha * yv[e];
+                store4(xr + c, v[i]);
+            }
+#pragma unroll
+            for (int e = 0; e < 4; ++e) ss += v[i][e] * v[i][e];
+        }
+    }
+    ss = block_sum(ss, red);
+    const float inv = 1.0f / sqrtf(ss / (float)d + eps);
+#pragma unroll
+    for (int i = 0; i < VPT; ++i) {
+        const int c = 4 * (threadIdx.x + i * blockDim.x);
+        if (c < d) {
+            float wv[4], o[4];
+            load4(w + c, wv);
+#pragma unroll
+            for (int e = 0; e < 4; ++e) o[e] = v[i][e] * inv * wv[e] * out_scale;
+            store4(out + (size_t)r * d + c, o);
+        }
+    }
+}
+
+// Threads per row and vectors per thread for the one-pass kernels; 0 if the row does not fit.
+static inline int norm_row_shape(int d, int* threads) {
+    if (d % 4) return 0;
+    const int vecs = d / 4;
+    int t = ((vecs + 63) / 64) * 64;
+    if (t > 1024) t = 1024;
+    *threads = t;
+    const int vpt = (vecs + t - 1) / t;
+    return vpt <= 4 ? vpt : 0;
+}
+
+template <typename TY, typename TO, bool ADD>
+static bool launch_norm_row(float* x, const int* rows, const TY* y, float alpha, const float* w, TO* out,
+                            int n_rows, int d, float eps, float out_scale, hipStream_t stream) {
+    int threads = 0;
+    const int vpt = norm_row_shape(d, &threads);
+    if (!vpt || ((uintptr_t)x & 15) || ((uintptr_t)w & 15) || ((uintptr_t)out & 7) || (ADD && ((uintptr_t)y & 7)))
+        return false;
+    dim3 grid(n_rows), block(threads);
+    switch (vpt) {
+    case 1: hipLaunchKernelGGL((norm_row_kernel<TY, TO, 1, ADD>), grid, block, 0, stream, x, rows, y, alpha, w, out, d, eps, out_scale); break;
+    case 2: hipLaunchKernelGGL((norm_row_kernel<TY, TO, 2, ADD>), grid, block, 0, stream, x, rows, y, alpha, w, out, d, eps, out_scale); break;
+    case 3: hipLaunchKernelGGL((norm_row_kernel<TY, TO, 3, ADD>), grid, block, 0, stream, x, rows, y, alpha, w, out, d, eps, out_scale); break;
+    default: hipLaunchKernelGGL((norm_row_kernel<TY, TO, 4, ADD>), grid, block, 0, stream, x, rows, y, alpha, w, out, d, eps, out_scale); break;
+    }
+    return true;
+}
+
 // ---------------------------------------------------------------------------
 // out[r, :] = x[rows ? rows[r] : r, :] * rsqrt(mean(x^2) + eps) * w * out_scale
 // ---------------------------------------------------------------------------
@@ -53,6 +143,10 @@ IC_EXPORT int ic_rmsnorm(const float* x, const int* rows, const float* w, void* 
                          int n_rows, int d, float eps, float out_scale, hipStream_t stream) {
     if (n_rows <= 0) return IC_OK;
     if (d <= 0) return IC_ERR_ARG;
+    if (out_dtype == IC_F32 && launch_norm_row<float, float, false>((float*)x, rows, (const float*)nullptr, 0.f, w, (float*)out, n_rows, d, eps, out_scale, stream))
+        return ic_launch_status();
+    if (out_dtype == IC_BF16 && launch_norm_row<float, bf16, false>((float*)x, rows, (const float*)nullptr, 0.f, w, (bf16*)out, n_rows, d, eps, out_scale, stream))
+        return ic_launch_status();
     dim3 grid(n_rows), block(d >= 1024 ? 256 : 128);
     if (out_dtype == IC_F32)
         hipLaunchKernelGGL(rmsnorm_kernel<float>, grid, block, 0, stream, x, rows, w, (float*)out, d, eps, out_scale);
@@ -89,6 +183,12 @@ IC_EXPORT int ic_add_rmsnorm(float* x, const void* y, int y_dtype, float alpha, 
                              void* out, int out_dtype, int T, int d, float eps, hipStream_t stream) {
     if (T <= 0) return IC_OK;
     if (d <= 0) return IC_ERR_ARG;
+    bool done = false;
+    if (y_dtype == IC_F32 && out_dtype == IC_F32) done = launch_norm_row<float, float, true>(x, nullptr, (const float*)y, alpha, w, (float*)out, T, d, eps, 1.f, stream);
+    else if (y_dtype == IC_BF16 && out_dtype == IC_BF16) done = launch_norm_row<bf16, bf16, true>(x, nullptr, (const bf16*)y, alpha, w, (bf16*)out, T, d, eps, 1.f, stream);
+    else if (y_dtype == IC_F32 && out_dtype == IC_BF16) done = launch_norm_row<float, bf16, true>(x, nullptr, (const float*)y, alpha, w, (bf16*)out, T, d, eps, 1.f, stream);
+    else if (y_dtype == IC_BF16 && out_dtype == IC_F32) done = launch_norm_row<bf16, float, true>(x, nullptr, (const bf16*)y, alpha, w, (float*)out, T, d, eps, 1.f, stream);
+    if (done) return ic_launch_status();
     dim3 grid(T), block(d >= 1024 ? 256 : 128);
     if (y_dtype == IC_F32 && out_dtype == IC_F32)
         hipLaunchKernelGGL((add_rmsnorm_kernel<float, float>), grid, block, 0, stream, x, (const float*)y, alpha, w, (float*)out, d, eps);

@@ -10,55 +10,47 @@
 // Cache layout of one layer: K and V planes [num_pages, n_kv_heads, page_size, head_dim].
 #include "common.h"
 
+constexpr int kRopeHeadsPerBlock = 4;
+
+// Grid (T, ceil((nh + 2 nkvh) / 4)), 256 threads: one wave per head of one token.
+// Heads 0..nh-1 are q, then nkvh k heads, then nkvh v heads.
 template <typename T>
-__global__ void rope_kv_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
-                               const float* __restrict__ cos_t, const float* __restrict__ sin_t,
-                               T* __restrict__ kcache, T* __restrict__ vcache,
-                               const int* __restrict__ slots,
-                               int row_stride, int nh, int nkvh, int dh, int rot, int page_size) {
+__global__ void __launch_bounds__(64 * kRopeHeadsPerBlock)
+rope_kv_kernel(T* __restrict__ qkv, const int* __restrict__ positions,
+               const float* __restrict__ cos_t, const float* __restrict__ sin_t,
+               T* __restrict__ kcache, T* __restrict__ vcache, const int* __restrict__ slots,
+               int row_stride, int nh, int nkvh, int dh, int rot, int page_size) {
     const int t = blockIdx.x;
-    T* row = qkv + (size_t)t * row_stride;
-    const int pos = positions[t];
+    const int head = blockIdx.y * kRopeHeadsPerBlock + (threadIdx.x >> 6);
+    const int lane = threadIdx.x & 63;
+    if (head >= nh + 2 * nkvh) return;
+    T* hp = qkv + (size_t)t * row_stride + (size_t)head * dh;
     const int half = rot >> 1;
+    T* dst = nullptr;                       // where the head goes in the cache (k and v heads)
+    if (head >= nh) {
+        const int slot = slots[t];
+        if (slot < 0) return;
+        const int pg = slot / page_size, off = slot - pg * page_size;
+        const int kh = (head < nh + nkvh) ? head - nh : head - nh - nkvh;
+        T* plane = (head < nh + nkvh) ? kcache : vcache;
+        dst = plane + (((size_t)pg * nkvh + kh) * page_size + off) * dh;
+    }
+    if (head >= nh + nkvh) {                // v: plain copy
+        for (int j = lane; j < dh; j += 64) dst[j] = hp[j];
+        return;
+    }
+    const int pos = positions[t];
     const float* cr = cos_t + (size_t)pos * half;
     const float* sr = sin_t + (size_t)pos * half;
-    const int slot = (nkvh > 0) ? slots[t] : -1;
-    const int pg = slot >= 0 ? slot / page_size : 0;
-    const int off = slot >= 0 ? slot - pg * page_size : 0;
-
-    // rotations of q and k heads
-    const int n_rot = (nh + nkvh) * half;
-    for (int i = threadIdx.x; i < n_rot; i += blockDim.x) {
-        const int head = i / half, j = i - head * half;
-        T* hp = row + (size_t)head * dh;
+    T* o = dst ? dst : hp;                  // q heads are rotated in place
+    for (int j = lane; j < half; j += 64) {
         const float a = to_f32(hp[j]), b = to_f32(hp[j + half]);
         const float c = cr[j], s = sr[j];
-        const T ra = from_f32<T>(a * c - b * s);
-        const T rb = from_f32<T>(a * s + b * c);
-        if (head < nh) {
-            hp[j] = ra;
-            hp[j + half] = rb;
-        } else if (slot >= 0) {
-            T* kp = kcache + (((size_t)pg * nkvh + (head - nh)) * page_size + off) * dh;
-            kp[j] = ra;
-            kp[j + half] = rb;
-        }
+        o[j] = from_f32<T>(a * c - b * s);
+        o[j + half] = from_f32<T>(a * s + b * c);
     }
-    if (nkvh == 0 || slot < 0) return;
-    // the part of each k head beyond the rotated dims passes through
-    const int tail = dh - rot;
-    if (tail > 0) {
-        for (int i = threadIdx.x; i < nkvh * tail; i += blockDim.x) {
-            const int kh = i / tail, j = rot + (i - kh * tail);
-            kcache[(((size_t)pg * nkvh + kh) * page_size + off) * dh + j] = row[(size_t)(nh + kh) * dh + j];
-        }
-    }
-    // values
-    const T* vsrc = row + (size_t)(nh + nkvh) * dh;
-    for (int i = threadIdx.x; i < nkvh * dh; i += blockDim.x) {
-        const int kh = i / dh, j = i - kh * dh;
-        vcache[(((size_t)pg * nkvh + kh) * page_size + off) * dh + j] = vsrc[i];
-    }
+    if (dst)                                // the part of a k head beyond the rotated dims passes through
+        for (int j = rot + lane; j < dh; j += 64) dst[j] = hp[j];
 }
 
 // qkv: [T, row_stride] with q heads first, then (if nkvh > 0) k heads, then v heads.
@@ -71,7 +63,8 @@ IC_EXPORT int ic_rope_kv_write(void* qkv, int dtype, const int* positions, const
     if (T <= 0) return IC_OK;
     if (dh <= 0 || rot < 0 || rot > dh || (rot & 1) || nh < 0 || nkvh < 0 || page_size <= 0) return IC_ERR_ARG;
     if (row_stride < (nh + 2 * nkvh) * dh) return IC_ERR_ARG;
-    dim3 grid(T), block(256);
+    if (T > 0x7fffffff || (nh + 2 * nkvh + kRopeHeadsPerBlock - 1) / kRopeHeadsPerBlock > 65535) return IC_ERR_ARG;
+    dim3 grid(T, (nh + 2 * nkvh + kRopeHeadsPerBlock - 1) / kRopeHeadsPerBlock), block(64 * kRopeHeadsPerBlock);
     if (dtype == IC_F32)
         hipLaunchKernelGGL(rope_kv_kernel<float>, grid, block, 0, stream, (float*)qkv, positions, cos_t, sin_t,
                            (float*)kcache, (float*)vcache, slots, row_stride, nh, nkvh, dh, rot, page_size);
