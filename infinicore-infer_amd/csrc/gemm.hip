@@ -36,19 +36,24 @@ __device__ __forceinline__ void load8(const uint16_t* __restrict__ p, int valid,
     }
 }
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED>
+template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, bool CSWIGLU>
 __global__ void __launch_bounds__(WPB * 64)
 gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C,
                     int M, int N, int K, int lda, int ldw, int ldc, float alpha) {
     __shared__ float red[WPB - 1][NT * MT][64][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
-    const int n0 = blockIdx.x * (16 * NT), m0 = blockIdx.y * (16 * MT);
+    // CSWIGLU: W = [gate rows (N/2); up rows (N/2)]; a block owns 16 gate rows and the matching
+    // 16 up rows and writes C[m][n] = up * silu(gate) for its 16 columns of the N/2 wide output.
+    const int NO = CSWIGLU ? N / 2 : N;                      // output columns
+    const int n0 = blockIdx.x * (CSWIGLU ? 16 : 16 * NT), m0 = blockIdx.y * (16 * MT);
 
     const uint16_t* wp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int nrow = (n0 + 16 * nt + r < N) ? n0 + 16 * nt + r : N - 1;
+        const int base = CSWIGLU ? n0 + nt * NO : n0 + 16 * nt;
+        const int lim = CSWIGLU ? (nt + 1) * NO : N;
+        const int nrow = (base + r < lim) ? base + r : lim - 1;
         wp[nt] = W + (size_t)nrow * ldw + 8 * kq;
     }
     const uint16_t* ap[MT];
@@ -107,6 +112,24 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     }
     __syncthreads();
     if (wave > 0) return;
+    if (CSWIGLU) {
+#pragma unroll
+        for (int mt = 0; mt < MT; ++mt) {
+            const int m = m0 + 16 * mt + r;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                float g = acc[0][mt][e], u = acc[NT - 1][mt][e];
+#pragma unroll
+                for (int w = 0; w < WPB - 1; ++w) { g += red[w][mt][lane][e]; u += red[w][(NT - 1) * MT + mt][lane][e]; }
+                // both projections are rounded to the output type first, as when they are stored
+                g = to_f32(from_f32<TC>(alpha * g));
+                u = to_f32(from_f32<TC>(alpha * u));
+                const int n = n0 + 4 * kq + e;
+                if (m < M && n < NO) C[(size_t)m * ldc + n] = from_f32<TC>(u * (g / (1.0f + expf(-g))));
+            }
+        }
+        return;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -128,11 +151,24 @@ static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int
                         int ldc, float alpha, bool aligned, hipStream_t stream) {
     dim3 grid((N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, false>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha);
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, false>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha);
+}
+
+// The gate/up projection with the activation in its epilogue: W [N, K] = [gate; up], C [M, N/2].
+template <typename TC, int WPB>
+static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
+                               int ldc, bool aligned, hipStream_t stream) {
+    dim3 grid((N / 2 + 15) / 16, (M + 15) / 16), block(WPB * 64);
+    if (aligned)
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, 2, true, true>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f);
+    else
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, 2, false, true>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f);
 }
 
 // NT weight tiles of 16 rows share one load of the A fragments; WPB waves split K.  Both are
@@ -192,13 +228,28 @@ IC_EXPORT int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype) {
     return a_dtype == IC_BF16 && w_dtype == IC_BF16 && (c_dtype == IC_F32 || c_dtype == IC_BF16);
 }
 
+// c_mode 0: C [M, N] = alpha * A W^T.  c_mode 1 (M <= 16, N even, alpha ignored): W = [gate; up] and
+// C [M, N/2] = up * silu(gate), both projections rounded to C's type before the activation.
 IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
-                         int M, int N, int K, int lda, int ldw, int ldc, float alpha, hipStream_t stream) {
+                         int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode,
+                         hipStream_t stream) {
     if (M <= 0 || N <= 0) return IC_OK;
-    if (K <= 0 || lda < K || ldw < K || ldc < N) return IC_ERR_ARG;
+    if (K <= 0 || lda < K || ldw < K || c_mode < 0 || c_mode > 1) return IC_ERR_ARG;
+    if (c_mode == 1 ? (M > 16 || (N & 1) || ldc < N / 2) : (ldc < N)) return IC_ERR_ARG;
     if (!ic_gemm_nt_supported(a_dtype, w_dtype, c_dtype)) return IC_ERR_UNSUPPORTED;
     if ((M + 63) / 64 > 65535) return IC_ERR_ARG;
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
+    if (c_mode == 1) {
+        const int tiles = (N / 2 + 15) / 16;
+        if (c_dtype == IC_F32) {
+            if (tiles < 300) launch_gemm_swiglu<float, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
+            else launch_gemm_swiglu<float, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
+        } else {
+            if (tiles < 300) launch_gemm_swiglu<bf16, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
+            else launch_gemm_swiglu<bf16, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
+        }
+        return ic_launch_status();
+    }
     if (c_dtype == IC_F32) dispatch_gemm<float>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
     else dispatch_gemm<bf16>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
     return ic_launch_status();

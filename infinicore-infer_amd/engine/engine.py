@@ -222,9 +222,12 @@ class Engine:
                 max_ctx = max(max_ctx, p0 + 1)
             else:
                 for o in range(0, n, self._tile_rows):
-                    tiles.extend((r, row0 + o, min(self._tile_rows, n - o), p0 + o))
+                    tiles.append((r, row0 + o, min(self._tile_rows, n - o), p0 + o))
             req_start.append(row0 + n)
         state_slots = [self.cache.state_slot(e.req_id) for e in entries]
+        # tiles that see the most keys go first, so the longest blocks do not form the tail
+        tiles.sort(key=lambda t: -(t[3] + t[2]))
+        tiles = [v for t in tiles for v in t]
 
         group_slots, group_tables, group_maxb = [], [], []
         for g in range(len(self.groups)):

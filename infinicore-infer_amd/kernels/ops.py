@@ -187,8 +187,8 @@ def attention_decode(q, out, kcache, vcache, block_tables, tok_list, n_tok, toke
         float(scale), int(window or 0), int(n_split), _stream()), "attention_decode")
 
 
-def attention_prefill_supported(dtype, head_dim: int) -> bool:
-    return bool(get_lib().ic_attn_prefill_supported(dtype_code(dtype), head_dim))
+def attention_prefill_supported(dtype, head_dim: int, page_size: int) -> bool:
+    return bool(get_lib().ic_attn_prefill_supported(dtype_code(dtype), head_dim, page_size))
 
 
 def attention_prefill_tile_rows() -> int:
@@ -234,14 +234,16 @@ def gemm_nt_supported(a_dtype, w_dtype, c_dtype) -> bool:
         return False
 
 
-def gemm_nt(a, w, out, alpha: float = 1.0):
-    """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation)."""
+def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False):
+    """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation).
+    swiglu_output (M <= 16): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate)."""
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
-    _need(w.shape[1] == K and tuple(out.shape) == (M, N), "gemm_nt: shape mismatch")
+    _need(w.shape[1] == K and tuple(out.shape) == (M, N // 2 if swiglu_output else N), "gemm_nt: shape mismatch")
+    _need(not swiglu_output or (M <= 16 and N % 2 == 0), "gemm_nt: fused activation needs M <= 16 and even N")
     _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm_nt: inner strides must be 1")
     check(get_lib().ic_gemm_nt(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
                                out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),
-                               out.stride(0), float(alpha), _stream()), "gemm_nt")
+                               out.stride(0), float(alpha), 1 if swiglu_output else 0, _stream()), "gemm_nt")
     return out

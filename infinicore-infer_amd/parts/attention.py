@@ -89,7 +89,7 @@ class Attention(Mixer):
         args = (self.nh, self.nkvh, self.dh, ctx.page_size)
         fast = rt.attention_impl == "auto"
         dec_ok = fast and ops.attention_decode_supported(rt.dtype, self.dh)
-        pre_ok = fast and ops.attention_prefill_supported(rt.dtype, self.dh)
+        pre_ok = fast and ops.attention_prefill_supported(rt.dtype, self.dh, ctx.page_size)
         n_dec, n_tiles = ctx.n_decode_rows, ctx.n_prefill_tiles
         use_dec = dec_ok and n_dec > 0 and (pre_ok or n_tiles == 0)
         use_pre = pre_ok and n_tiles > 0 and (dec_ok or n_dec == 0)

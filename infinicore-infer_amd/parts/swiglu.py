@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import FeedForward, register_part
-from .linear import linear
+from .linear import FEW_ROWS, linear
 
 
 @register_part("feed_forward", "swiglu")
@@ -43,10 +43,15 @@ class SwiGLU(FeedForward):
     def forward(self, h, ctx):
         rt = self.runtime
         T = h.shape[0]
-        gate_up = ctx.ws.buffer("gate_up", (T, 2 * self.intermediate_size), rt.dtype)
-        linear(h, self.w_gate_up, gate_up, rt.gemm_impl)
         act = ctx.ws.buffer("ffn_act", (T, self.intermediate_size), rt.dtype)
-        ops.swiglu(gate_up, act)
+        if (T <= FEW_ROWS and rt.gemm_impl == "auto" and self.w_gate_up.dtype == h.dtype
+                and ops.gemm_nt_supported(h.dtype, self.w_gate_up.dtype, act.dtype)):
+            # few rows: the activation is the epilogue of the gate/up projection
+            ops.gemm_nt(h, self.w_gate_up, act, swiglu_output=True)
+        else:
+            gate_up = ctx.ws.buffer("gate_up", (T, 2 * self.intermediate_size), rt.dtype)
+            linear(h, self.w_gate_up, gate_up, rt.gemm_impl)
+            ops.swiglu(gate_up, act)
         y = ctx.ws.buffer("ffn_out", (T, self.hidden_size), rt.dtype)
         linear(act, self.w_down, y, rt.gemm_impl)
         return y

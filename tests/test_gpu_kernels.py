@@ -381,3 +381,18 @@ def test_sampling_distribution():
     expect = torch.softmax(row.double(), 0) * n
     chi2 = float(((counts - expect) ** 2 / expect).sum())
     assert chi2 < 40.0, "chi-square %.1f over %d bins" % (chi2, V)       # 11 dof: p(chi2 > 40) < 1e-4
+
+
+@pytest.mark.parametrize("cdtype", DT)
+@pytest.mark.parametrize("M,di,K", [(1, 344, 200), (8, 5760, 2304), (16, 256, 96), (5, 130, 100), (3, 3840, 1536)])
+def test_gemm_nt_with_swiglu_output(cdtype, M, di, K):
+    """The gate/up projection with the activation in its epilogue equals the plain product
+    followed by the SwiGLU kernel."""
+    g = torch.Generator().manual_seed(21)
+    h = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(2 * di, K, generator=g) * 0.1).to(torch.bfloat16)
+    out = torch.empty(M, di, dtype=cdtype, device=DEV)
+    _ops().gemm_nt(h.to(DEV), w.to(DEV), out, swiglu_output=True)
+    rnd = P.round_bf16 if cdtype == torch.bfloat16 else (lambda t: t)
+    gu = rnd(P.plain_linear(h, w))
+    _close(out, P.plain_swiglu(gu[:, :di], gu[:, di:]), cdtype, factor=2 if cdtype == torch.bfloat16 else 50)
