@@ -15,24 +15,28 @@
 constexpr int kDecThreads = 256;
 constexpr int kDecWaves = kDecThreads / 64;
 constexpr int kDecUnroll = 4;
+constexpr int kDecMaxPages = 1024;   // page ids of one block's keys staged in LDS (else read from memory)
 
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {
     static constexpr int N = 4;
-    __device__ static void load(const float* p, float* o) {
-        const float4 v = *reinterpret_cast<const float4*>(p);
-        o[0] = v.x; o[1] = v.y; o[2] = v.z; o[3] = v.w;
+    __device__ static uint4 raw(const float* p) { return *reinterpret_cast<const uint4*>(p); }
+    __device__ static void unpack(const uint4& v, float* o) {
+        o[0] = __uint_as_float(v.x); o[1] = __uint_as_float(v.y);
+        o[2] = __uint_as_float(v.z); o[3] = __uint_as_float(v.w);
     }
+    __device__ static void load(const float* p, float* o) { unpack(raw(p), o); }
 };
 template <> struct Vec16<bf16> {
     static constexpr int N = 8;
-    __device__ static void load(const bf16* p, float* o) {
-        const uint4 v = *reinterpret_cast<const uint4*>(p);
+    __device__ static uint4 raw(const bf16* p) { return *reinterpret_cast<const uint4*>(p); }
+    __device__ static void unpack(const uint4& v, float* o) {
         o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
         o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
         o[4] = __uint_as_float(v.z << 16); o[5] = __uint_as_float(v.z & 0xffff0000u);
         o[6] = __uint_as_float(v.w << 16); o[7] = __uint_as_float(v.w & 0xffff0000u);
     }
+    __device__ static void load(const bf16* p, float* o) { unpack(raw(p), o); }
 };
 
 // merge running-softmax state b into a
@@ -63,6 +67,7 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
 
     __shared__ float sm_acc[kDecWaves][GQ][DH];
     __shared__ float sm_ml[kDecWaves][GQ][2];
+    __shared__ int pages[kDecMaxPages];
 
     const int split = blockIdx.x, kvh = blockIdx.y, n = blockIdx.z;
     const int t = tok_list ? tok_list[n] : n;
@@ -80,6 +85,24 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
     const int sub = lane % LPK;                   // which 16-byte slice of the row
     const int grp = lane / LPK;                   // which key of the wave's step
     const size_t head_stride = (size_t)page_size * DH;
+    const size_t page_stride = (size_t)nkvh * head_stride;
+    const T* kbase = kcache + (size_t)kvh * head_stride + sub * VEC;
+    const T* vbase = vcache + (size_t)kvh * head_stride + sub * VEC;
+
+    // page ids of this block's keys, staged once: the loop then needs one memory hop per key
+    const int page_lo = lo / page_size;
+    const int n_pages = (hi > lo) ? (hi - 1) / page_size - page_lo + 1 : 0;
+    const bool staged = n_pages <= kDecMaxPages;
+    if (staged)
+        for (int i = threadIdx.x; i < n_pages; i += kDecThreads) pages[i] = bt[page_lo + i];
+    __syncthreads();
+
+    // element offset of a key's row piece in a plane
+    auto row_of = [&](int key) -> size_t {
+        const int lp = key / page_size;
+        const int pg = staged ? pages[lp - page_lo] : bt[lp];
+        return (size_t)pg * page_stride + (size_t)(key - lp * page_size) * DH;
+    };
 
     for (int h0 = 0; h0 < g; h0 += GQ) {
         float qv[GQ][VEC], acc[GQ][VEC], m[GQ], l[GQ];
@@ -92,20 +115,26 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
             for (int i = 0; i < VEC; ++i) { qv[j][i] *= scale; acc[j][i] = 0.f; }
         }
 
-        for (int kb = lo + wave * KPW + grp; kb < hi; kb += kDecUnroll * KPB) {
-            float kf[kDecUnroll][VEC], vf[kDecUnroll][VEC];
-            bool ok[kDecUnroll];
+        // keys kb, kb + KPB, ... of one step; the next step's loads are issued before this one is used
+        uint4 kr[2][kDecUnroll], vr[2][kDecUnroll];
+        auto issue = [&](int kb, uint4* kk, uint4* vv) {
 #pragma unroll
             for (int u = 0; u < kDecUnroll; ++u) {
                 const int key = kb + u * KPB;
-                ok[u] = key < hi;
-                if (ok[u]) {
-                    const int pg = bt[key / page_size];
-                    const int off = key % page_size;
-                    const size_t base = ((size_t)pg * nkvh + kvh) * head_stride + (size_t)off * DH + sub * VEC;
-                    Vec16<T>::load(kcache + base, kf[u]);
-                    Vec16<T>::load(vcache + base, vf[u]);
+                if (key < hi) {
+                    const size_t off = row_of(key);
+                    kk[u] = Vec16<T>::raw(kbase + off);
+                    vv[u] = Vec16<T>::raw(vbase + off);
                 }
+            }
+        };
+        auto consume = [&](int kb, const uint4* kk, const uint4* vv) {
+            float kf[kDecUnroll][VEC];
+            bool ok[kDecUnroll];
+#pragma unroll
+            for (int u = 0; u < kDecUnroll; ++u) {
+                ok[u] = kb + u * KPB < hi;
+                if (ok[u]) Vec16<T>::unpack(kk[u], kf[u]);
             }
 #pragma unroll
             for (int j = 0; j < GQ; ++j) {
@@ -131,15 +160,26 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
 #pragma unroll
                 for (int u = 0; u < kDecUnroll; ++u) {
                     if (ok[u]) {
+                        float vf[VEC];
+                        Vec16<T>::unpack(vv[u], vf);
                         const float p = expf(s[u] - mx);
                         lsum += p;
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) acc[j][i] += p * vf[u][i];
+                        for (int i = 0; i < VEC; ++i) acc[j][i] += p * vf[i];
                     }
                 }
                 l[j] = lsum;
                 m[j] = mx;
             }
+        };
+        constexpr int STEP = kDecUnroll * KPB;
+        const int kb0 = lo + wave * KPW + grp;
+        issue(kb0, kr[0], vr[0]);
+        for (int kb = kb0; kb < hi; kb += 2 * STEP) {
+            issue(kb + STEP, kr[1], vr[1]);
+            consume(kb, kr[0], vr[0]);
+            issue(kb + 2 * STEP, kr[0], vr[0]);
+            consume(kb + STEP, kr[1], vr[1]);
         }
 
         // merge the lane groups of the wave (lanes with the same `sub`)

@@ -85,12 +85,16 @@ class StepContext:
         return v
 
     def decode_splits(self, n_kv_heads: int, window: int = 0) -> int:
-        """How many ways to split the keys of single-token rows so that the grid
-        fills the chip: enough blocks for ~4 per compute unit, at least 256 keys each."""
+        """How many ways to split the keys of single-token rows.  From a sweep on MI355X: few
+        rows want about 2.25 blocks per compute unit however short the loops get; many rows want
+        about 9 per unit; a split never gets fewer than 64 keys."""
         if self.fixed_decode_splits is not None:
             return self.fixed_decode_splits
         keys = self.max_context if not window else min(self.max_context, window)
-        blocks = max(1, self.n_decode_rows * n_kv_heads)
-        want = max(1, (4 * self.cu_count + blocks - 1) // blocks)
-        most = max(1, keys // 256)
-        return int(max(1, min(want, most, 64)))
+        base = max(1, self.n_decode_rows * n_kv_heads)
+        few = (9 * self.cu_count + 3) // 4
+        if base < few:
+            want = (few + base - 1) // base
+        else:
+            want = max(1, (9 * self.cu_count + base // 2) // base)
+        return int(max(1, min(want, max(1, keys // 64), 64)))
