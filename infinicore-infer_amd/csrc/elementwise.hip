@@ -243,12 +243,38 @@ __global__ void swiglu_kernel(const T* __restrict__ gu, T* __restrict__ out, int
     }
 }
 
+// eight elements per thread (di % 8 == 0, 16-byte aligned rows)
+__global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict__ out, int di, size_t n8) {
+    size_t i = (size_t)blockIdx.x * blockDim.x + threadIdx.x;
+    const size_t step = (size_t)gridDim.x * blockDim.x;
+    const int per_row = di >> 3;
+    for (; i < n8; i += step) {
+        const size_t t = i / per_row;
+        const int j = (int)(i - t * per_row) << 3;
+        const bf16* gp = gu + t * 2 * (size_t)di + j;
+        float g[8], u[8], o[8];
+        load4(gp, g); load4(gp + 4, g + 4);
+        load4(gp + di, u); load4(gp + di + 4, u + 4);
+#pragma unroll
+        for (int e = 0; e < 8; ++e) o[e] = u[e] * (g[e] / (1.0f + expf(-g[e])));
+        bf16* op = out + t * (size_t)di + j;
+        store4(op, o); store4(op + 4, o + 4);
+    }
+}
+
 IC_EXPORT int ic_swiglu(const void* gate_up, void* out, int dtype, int T, int di, hipStream_t stream) {
     if (T <= 0) return IC_OK;
     if (di <= 0) return IC_ERR_ARG;
     const size_t n = (size_t)T * di;
     int blocks = (int)((n + 255) / 256);
     if (blocks > 16384) blocks = 16384;
+    if (dtype == IC_BF16 && di % 8 == 0 && !((uintptr_t)gate_up & 15) && !((uintptr_t)out & 15)) {
+        const size_t n8 = n / 8;
+        int b8 = (int)((n8 + 255) / 256);
+        if (b8 > 65536) b8 = 65536;
+        hipLaunchKernelGGL(swiglu_vec8_kernel, dim3(b8), dim3(256), 0, stream, (const bf16*)gate_up, (bf16*)out, di, n8);
+        return ic_launch_status();
+    }
     if (dtype == IC_F32)
         hipLaunchKernelGGL(swiglu_kernel<float>, dim3(blocks), dim3(256), 0, stream, (const float*)gate_up, (float*)out, di, n);
     else if (dtype == IC_BF16)
