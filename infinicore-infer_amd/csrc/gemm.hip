@@ -159,15 +159,15 @@ static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int
 }
 
 // The gate/up projection with the activation in its epilogue: W [N, K] = [gate; up], C [M, N/2].
-template <typename TC, int WPB>
+template <typename TC, int WPB, int UN = 2>
 static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
                                int ldc, bool aligned, hipStream_t stream) {
     dim3 grid((N / 2 + 15) / 16, (M + 15) / 16), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, 2, true, true>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, true, true>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f);
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, 2, false, true>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, false, true>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f);
 }
 
@@ -211,8 +211,16 @@ static int launch_cfg_m(const void* A, const void* W, void* C, int M, int N, int
 IC_EXPORT int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda,
                              int ldw, int ldc, float alpha, int nt, int wpb, int unroll, hipStream_t stream) {
     if (M <= 0 || N <= 0) return IC_OK;
-    if (K <= 0 || lda < K || ldw < K || ldc < N || c_dtype != IC_BF16) return IC_ERR_ARG;
+    if (K <= 0 || lda < K || ldw < K || c_dtype != IC_BF16) return IC_ERR_ARG;
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
+    if (nt == 0) {                                  // nt == 0: the variant with SwiGLU in the epilogue
+        if (M > 16 || (N & 1) || ldc < N / 2) return IC_ERR_ARG;
+#define IC_SW(WPB, UN) if (wpb == WPB && unroll == UN) { launch_gemm_swiglu<bf16, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream); return ic_launch_status(); }
+        IC_SW(4, 2) IC_SW(4, 4) IC_SW(8, 2) IC_SW(8, 4) IC_SW(16, 2) IC_SW(16, 4)
+#undef IC_SW
+        return IC_ERR_UNSUPPORTED;
+    }
+    if (ldc < N) return IC_ERR_ARG;
     int st = IC_ERR_UNSUPPORTED;
 #define IC_CFG(NT, WPB, UN) \
     if (nt == NT && wpb == WPB && unroll == UN) st = launch_cfg_m<bf16, NT, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);

@@ -180,6 +180,60 @@ sample_kernel(const float* __restrict__ logits, long long row_stride, int V,
     }
 }
 
+// ---- argmax in two stages: many blocks per row, then one wave per row --------------------------
+constexpr int kArgmaxChunks = 64;
+
+__device__ __forceinline__ void argmax_merge(float& best, int& besti, float ob, int oi) {
+    if (ob > best || (ob == best && oi < besti)) { best = ob; besti = oi; }
+}
+
+__global__ void __launch_bounds__(256)
+argmax_partial_kernel(const float* __restrict__ logits, long long row_stride, int V,
+                      float* __restrict__ pval, int* __restrict__ pidx) {
+    __shared__ float red[4];
+    __shared__ int redi[4];
+    const int r = blockIdx.y, c = blockIdx.x, tid = threadIdx.x;
+    const float* row = logits + (size_t)r * row_stride;
+    const int per = (V + kArgmaxChunks - 1) / kArgmaxChunks;
+    const int lo = c * per, hi = (lo + per < V) ? lo + per : V;
+    float best = -INFINITY;
+    int besti = 0x7fffffff;
+    for (int i = lo + tid; i < hi; i += 256) argmax_merge(best, besti, row[i], i);
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) argmax_merge(best, besti, __shfl_xor(best, o, kWave), __shfl_xor(besti, o, kWave));
+    if ((tid & 63) == 0) { red[tid >> 6] = best; redi[tid >> 6] = besti; }
+    __syncthreads();
+    if (tid == 0) {
+        for (int w = 1; w < 4; ++w) argmax_merge(best, besti, red[w], redi[w]);
+        pval[r * kArgmaxChunks + c] = best;
+        pidx[r * kArgmaxChunks + c] = besti;
+    }
+}
+
+__global__ void __launch_bounds__(64)
+argmax_final_kernel(const float* __restrict__ pval, const int* __restrict__ pidx, int* __restrict__ out) {
+    const int r = blockIdx.x, lane = threadIdx.x;
+    float best = pval[r * kArgmaxChunks + lane];
+    int besti = pidx[r * kArgmaxChunks + lane];
+#pragma unroll
+    for (int o = 32; o > 0; o >>= 1) argmax_merge(best, besti, __shfl_xor(best, o, kWave), __shfl_xor(besti, o, kWave));
+    if (lane == 0) out[r] = besti;
+}
+
+// Greedy choice for every row (lowest index among equal maxima).  scratch_val / scratch_idx:
+// n_rows * 64 floats / ints.
+IC_EXPORT int ic_argmax(const float* logits, long long row_stride, int n_rows, int V, float* scratch_val,
+                        int* scratch_idx, int* out, hipStream_t stream) {
+    if (n_rows <= 0) return IC_OK;
+    if (V <= 0 || row_stride < V || n_rows > 65535) return IC_ERR_ARG;
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxChunks, n_rows), dim3(256), 0, stream, logits,
+                       row_stride, V, scratch_val, scratch_idx);
+    int st = ic_launch_status();
+    if (st) return st;
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(64), 0, stream, scratch_val, scratch_idx, out);
+    return ic_launch_status();
+}
+
 // logits [n_rows, V] float32 with row stride `row_stride` elements.  temperature,
 // top_k, top_p, uniform: per-row device arrays; passing temperature == nullptr
 // means argmax for every row.

@@ -329,6 +329,31 @@ class Engine:
         self.graph_replays += 1
         return g.logits
 
+    # ---- library products ----------------------------------------------------------------------------
+    def tune_library_products(self, token_counts: Sequence[int], max_ms_per_shape: int = 300) -> None:
+        """Let the library pick its fastest matrix-product kernel for prompt portions of the given
+        token counts (PyTorch's tunable-op mechanism over hipBLASLt and rocBLAS): one dummy step per
+        count is run with tuning on, then tuning is switched off again, so other shapes keep the
+        library's default choice and cost nothing.  Optional; results live for this process."""
+        import torch.cuda.tunable as tunable
+        tunable.enable(True)
+        tunable.tuning_enable(True)
+        tunable.set_max_tuning_duration(int(max_ms_per_shape))
+        if hasattr(tunable, "write_file_on_exit"):
+            tunable.write_file_on_exit(False)
+        else:                                     # keep the results file out of the working directory
+            import os
+            import tempfile
+            tunable.set_filename(os.path.join(tempfile.gettempdir(), "infinicore_infer_amd-tunable-%d.csv" % os.getpid()))
+        try:
+            for n in token_counts:
+                rid = ("tune", n)
+                self.step([StepEntry(rid, [0] * int(n), [int(n) - 1])])
+                self.free(rid)
+            torch.cuda.synchronize()
+        finally:
+            tunable.tuning_enable(False)
+
     # ---- sampling --------------------------------------------------------------------------------------
     def sample(self, logits, temperature=None, top_k=None, top_p=None, uniform=None) -> List[int]:
         """Tokens for the rows of ``logits``.  With ``temperature`` None every row is
@@ -336,7 +361,8 @@ class Engine:
         R = logits.shape[0]
         out = self.ws.buffer("sampled", (R,), torch.int32)
         if temperature is None:
-            ops.sample(logits, out)
+            ops.argmax(logits, out, self.ws.buffer("argmax_val", (64 * R,), torch.float32),
+                       self.ws.buffer("argmax_idx", (64 * R,), torch.int32))
         else:
             f = torch.tensor([list(temperature), list(top_p), list(uniform)], dtype=torch.float32).to(self.device)
             k = torch.tensor(list(top_k), dtype=torch.int32).to(self.device)

@@ -227,6 +227,21 @@ def sample(logits, out, temperature=None, top_k=None, top_p=None, uniform=None):
     return out
 
 
+def argmax(logits, out, scratch_val, scratch_idx):
+    """out[r] = index of the largest logit of row r (the lowest index among equals), in two
+    stages; scratch_val float32 and scratch_idx int32 of at least 64 * rows elements."""
+    _dev(logits, out, scratch_val, scratch_idx)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax: logits must be float32 rows")
+    _i32(out, "out")
+    _i32(scratch_idx, "scratch_idx")
+    _need(out.numel() >= R and scratch_val.dtype == torch.float32 and scratch_val.is_contiguous()
+          and scratch_val.numel() >= 64 * R and scratch_idx.numel() >= 64 * R, "argmax: buffers too small")
+    check(get_lib().ic_argmax(logits.data_ptr(), logits.stride(0), R, V, scratch_val.data_ptr(),
+                              scratch_idx.data_ptr(), out.data_ptr(), _stream()), "argmax")
+    return out
+
+
 def gemm_nt_supported(a_dtype, w_dtype, c_dtype) -> bool:
     try:
         return bool(get_lib().ic_gemm_nt_supported(dtype_code(a_dtype), dtype_code(w_dtype), dtype_code(c_dtype)))

@@ -361,9 +361,14 @@ def test_sampling(V):
         want = P.plain_sample(logits[r], float(temps[r]), int(ks[r]), float(ps[r]), float(us[r]))
         assert got[r] == want, "row %d (T=%g k=%d p=%g u=%g): got %d, plain %d" % (
             r, temps[r], ks[r], ps[r], us[r], got[r], want)
-    # argmax for every row when no temperature is given
+    # argmax for every row when no temperature is given, in one kernel and in two stages
+    want = [int(torch.argmax(logits[r])) for r in range(R)]
+    want[0] = 10
     ops.sample(logits.to(DEV), out)
-    assert out.cpu().tolist() == [int(torch.argmax(logits[r])) for r in range(R)]
+    assert out.cpu().tolist() == want
+    out.zero_()
+    ops.argmax(logits.to(DEV), out, torch.empty(64 * R, device=DEV), torch.empty(64 * R, dtype=torch.int32, device=DEV))
+    assert out.cpu().tolist() == want
 
 
 def test_sampling_distribution():
