@@ -84,6 +84,7 @@ class RequestEntry:
     length: int = 0                                  # tokens whose keys are in the cache
     tables: List[List[int]] = field(default_factory=list)   # per group: page id per logical page, -1 = given back
     first_live: List[int] = field(default_factory=list)     # per group: first logical page still held
+    serial: int = 0                                  # admission number: tells two lives of one request id apart
 
 
 class CacheManager:
@@ -102,6 +103,7 @@ class CacheManager:
         self.pools = [PagePool(n) for n in num_pages]
         self.slots = SlotPool(max_requests)
         self.requests: Dict[object, RequestEntry] = {}
+        self._admissions = 0
 
     # ---- admission ------------------------------------------------------------
     def has_request(self, req_id) -> bool:
@@ -117,8 +119,10 @@ class CacheManager:
         if self.slots.n_free == 0:
             raise OutOfPages("no free state slot (max_requests = %d)" % self.max_requests)
         slot = self.slots.alloc()
+        self._admissions += 1
         self.requests[req_id] = RequestEntry(
-            state_slot=slot, tables=[[] for _ in self.groups], first_live=[0] * len(self.groups))
+            state_slot=slot, tables=[[] for _ in self.groups], first_live=[0] * len(self.groups),
+            serial=self._admissions)
         return slot
 
     # ---- growth ---------------------------------------------------------------

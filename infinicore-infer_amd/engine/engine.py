@@ -314,15 +314,12 @@ class Engine:
         if g is None:
             g = _DecodeGraph(self, R, bucket)
             self._graphs[key] = g
-        host = self._ring.get(g.total)
-        flat = g.fill(self, entries, starts)
-        host[:g.total] = torch.tensor(flat, dtype=torch.int32)
-        g.meta[:g.total].copy_(host[:g.total], non_blocking=True)
-        self._ring.mark()
+        g.fill(self, entries, starts)
+        g.meta.copy_(g.host, non_blocking=True)
+        g.copied.record()
         g.ctx.max_position = max(starts)
         g.ctx.req_pos = list(starts)
         g.ctx.req_ids = [e.req_id for e in entries]
-        g.ctx.host_state_slots = flat[g.off["state_slots"]:g.off["state_slots"] + R]
         if g.graph is None:
             g.capture(self)
         g.graph.replay()
@@ -391,6 +388,14 @@ class _DecodeGraph:
         self.total = total
         self.sizes = sizes
         self.meta = torch.zeros(total, dtype=torch.int32, device=engine.device)
+        # the host image of ``meta``: pinned, kept between steps and changed only where the step differs
+        self.host = torch.zeros(total, dtype=torch.int32, pin_memory=True)
+        self.np = self.host.numpy()
+        self.copied = torch.cuda.Event()
+        self.copied.record()
+        self.np[self.off["token_req"]:self.off["token_req"] + R] = range(R)
+        self.np[self.off["want_rows"]:self.off["want_rows"] + R] = range(R)
+        self._row_keys = [[None] * R for _ in range(ng)]
         self.graph = None
         self.logits = None
 
@@ -420,22 +425,30 @@ class _DecodeGraph:
         self.ctx = ctx
 
     def fill(self, engine, entries, starts):
-        R, ps = self.R, engine.page_size
-        flat = [0] * self.total
-        o = self.off
+        """Write this step's integers into the pinned image.  Block-table rows are rewritten
+        only when the request in that row, its page count or its first live page changed."""
+        self.copied.synchronize()                   # the last copy out of the image is done
+        ps, a, o = engine.page_size, self.np, self.off
+        cache = engine.cache
+        slots = []
         for r, (e, p0) in enumerate(zip(entries, starts)):
-            flat[o["tokens"] + r] = int(e.tokens[0])
-            flat[o["positions"] + r] = p0
-            flat[o["token_req"] + r] = r
-            flat[o["state_slots"] + r] = engine.cache.state_slot(e.req_id)
-            flat[o["want_rows"] + r] = r
+            req = cache.requests[e.req_id]
+            a[o["tokens"] + r] = e.tokens[0]
+            a[o["positions"] + r] = p0
+            a[o["state_slots"] + r] = req.state_slot
+            slots.append(req.state_slot)
             for g in range(len(engine.groups)):
-                table = engine.cache.block_table(e.req_id, g)
-                flat[o["slots%d" % g] + r] = table[p0 // ps] * ps + p0 % ps
-                base = o["tables%d" % g] + r * self.maxb
-                for j, p in enumerate(table):
-                    flat[base + j] = p if p > 0 else 0
-        return flat
+                table = req.tables[g]
+                a[o["slots%d" % g] + r] = table[p0 // ps] * ps + p0 % ps
+                key = (req.serial, len(table), req.first_live[g])
+                if self._row_keys[g][r] != key:
+                    base = o["tables%d" % g] + r * self.maxb
+                    a[base:base + len(table)] = table
+                    if req.first_live[g]:
+                        a[base:base + req.first_live[g]] = 0     # pages given back are never read; keep the index valid
+                    a[base + len(table):base + self.maxb] = 0
+                    self._row_keys[g][r] = key
+        self.ctx.host_state_slots = slots
 
     def capture(self, engine):
         """Run the step once eagerly (every buffer then exists and the result is
