@@ -36,22 +36,53 @@ __device__ __forceinline__ void load8(const uint16_t* __restrict__ p, int valid,
     }
 }
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, bool CSWIGLU>
+// What the fused projection + rotary + cache-write epilogue needs beside the product.
+struct RopeEpilogue {
+    const int* positions;      // [M]
+    const int* slots;          // [M] token slot in the cache (page * page_size + offset), < 0: no write
+    const float* cos_t;        // [max_pos, dh/2]
+    const float* sin_t;
+    void* kcache;              // [pages, nkvh, page_size, dh]
+    void* vcache;
+    int nh, nkvh, dh, page_size;
+};
+
+template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI>
 __global__ void __launch_bounds__(WPB * 64)
 gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C,
-                    int M, int N, int K, int lda, int ldw, int ldc, float alpha) {
+                    int M, int N, int K, int lda, int ldw, int ldc, float alpha, RopeEpilogue rope) {
+    constexpr bool CSWIGLU = (EPI == 1);
+    constexpr bool CROPE = (EPI == 2);
     __shared__ float red[WPB - 1][NT * MT][64][4];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
     // CSWIGLU: W = [gate rows (N/2); up rows (N/2)]; a block owns 16 gate rows and the matching
     // 16 up rows and writes C[m][n] = up * silu(gate) for its 16 columns of the N/2 wide output.
+    // CROPE: W = [q heads; k heads; v heads] (rows of dh).  A block owns 16 rows j.. of one q or k
+    // head and the 16 rows j + dh/2.. that rotate with them, or 32 consecutive rows of a v head.
     const int NO = CSWIGLU ? N / 2 : N;                      // output columns
-    const int n0 = blockIdx.x * (CSWIGLU ? 16 : 16 * NT), m0 = blockIdx.y * (16 * MT);
+    int n0 = blockIdx.x * (CSWIGLU ? 16 : 16 * NT);
+    const int m0 = blockIdx.y * (16 * MT);
+    int rope_head = 0, rope_j = 0;                           // CROPE: head and first index in the head
+    bool rope_is_v = false;
+    if (CROPE) {
+        const int half = rope.dh >> 1, pt = half >> 4, n_rot = (rope.nh + rope.nkvh) * pt;
+        const int p = blockIdx.x;
+        if (p < n_rot) { rope_head = p / pt; rope_j = 16 * (p - rope_head * pt); }
+        else {
+            const int vt = rope.dh >> 5, pv = p - n_rot;
+            rope_is_v = true;
+            rope_head = rope.nh + rope.nkvh + pv / vt;
+            rope_j = 32 * (pv % vt);
+        }
+        n0 = rope_head * rope.dh + rope_j;
+    }
 
     const uint16_t* wp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        const int base = CSWIGLU ? n0 + nt * NO : n0 + 16 * nt;
+        int base = CSWIGLU ? n0 + nt * NO : n0 + 16 * nt;
+        if (CROPE && nt == 1 && !rope_is_v) base = n0 + (rope.dh >> 1);
         const int lim = CSWIGLU ? (nt + 1) * NO : N;
         const int nrow = (base + r < lim) ? base + r : lim - 1;
         wp[nt] = W + (size_t)nrow * ldw + 8 * kq;
@@ -130,6 +161,46 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         }
         return;
     }
+    if (CROPE) {
+        const int m = m0 + r;                           // MT == 1
+        if (m >= M) return;
+        float v0[4], v1[4];
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float a0 = acc[0][0][e], a1 = acc[NT - 1][0][e];
+#pragma unroll
+            for (int w = 0; w < WPB - 1; ++w) { a0 += red[w][0][lane][e]; a1 += red[w][NT - 1][lane][e]; }
+            v0[e] = to_f32(from_f32<TC>(a0));           // the projection is rounded to its type first, as when stored
+            v1[e] = to_f32(from_f32<TC>(a1));
+        }
+        const int half = rope.dh >> 1;
+        const int slot = rope.slots[m];
+        const int pg = slot >= 0 ? slot / rope.page_size : 0, off = slot >= 0 ? slot - pg * rope.page_size : 0;
+        const int jj = rope_j + 4 * kq;                 // first of this lane's four indices in the head
+        if (rope_is_v) {
+            if (slot < 0) return;
+            const int kh = rope_head - rope.nh - rope.nkvh;
+            TC* dst = (TC*)rope.vcache + (((size_t)pg * rope.nkvh + kh) * rope.page_size + off) * rope.dh;
+#pragma unroll
+            for (int e = 0; e < 4; ++e) { dst[jj + e] = from_f32<TC>(v0[e]); dst[jj + 16 + e] = from_f32<TC>(v1[e]); }
+            return;
+        }
+        const float4 c = *reinterpret_cast<const float4*>(rope.cos_t + (size_t)rope.positions[m] * half + jj);
+        const float4 s = *reinterpret_cast<const float4*>(rope.sin_t + (size_t)rope.positions[m] * half + jj);
+        const float cc[4] = {c.x, c.y, c.z, c.w}, ss[4] = {s.x, s.y, s.z, s.w};
+        TC* dst;
+        if (rope_head < rope.nh) dst = C + (size_t)m * ldc + (size_t)rope_head * rope.dh;
+        else {
+            if (slot < 0) return;
+            dst = (TC*)rope.kcache + (((size_t)pg * rope.nkvh + (rope_head - rope.nh)) * rope.page_size + off) * rope.dh;
+        }
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            dst[jj + e] = from_f32<TC>(v0[e] * cc[e] - v1[e] * ss[e]);
+            dst[jj + half + e] = from_f32<TC>(v0[e] * ss[e] + v1[e] * cc[e]);
+        }
+        return;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -151,11 +222,11 @@ static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int
                         int ldc, float alpha, bool aligned, hipStream_t stream) {
     dim3 grid((N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, false>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha);
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, 0>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{});
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, false>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha);
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, 0>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{});
 }
 
 // The gate/up projection with the activation in its epilogue: W [N, K] = [gate; up], C [M, N/2].
@@ -164,11 +235,11 @@ static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int
                                int ldc, bool aligned, hipStream_t stream) {
     dim3 grid((N / 2 + 15) / 16, (M + 15) / 16), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, true, true>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f);
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, true, 1>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{});
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, false, true>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f);
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, false, 1>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{});
 }
 
 // NT weight tiles of 16 rows share one load of the A fragments; WPB waves split K.  Both are
@@ -260,5 +331,33 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
     }
     if (c_dtype == IC_F32) dispatch_gemm<float>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
     else dispatch_gemm<bf16>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
+    return ic_launch_status();
+}
+
+// The fused QKV projection of few rows (M <= 16) with the rotary encoding and the cache write in
+// its epilogue: q heads land rotated in C[M, >= nh*dh] (row stride ldc), k heads rotated and v
+// heads as they are in the token's cache slot.  bfloat16 throughout; full rotary (rot == dh);
+// dh a multiple of 32.  W: [(nh + 2 nkvh) * dh, K].
+IC_EXPORT int ic_gemm_qkv_rope_supported(int dtype, int dh) { return dtype == IC_BF16 && dh >= 32 && dh % 32 == 0; }
+
+IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc,
+                               const int* positions, const int* slots, const float* cos_t, const float* sin_t,
+                               void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size,
+                               hipStream_t stream) {
+    if (M <= 0) return IC_OK;
+    if (M > 16 || K <= 0 || lda < K || ldw < K || nh <= 0 || nkvh <= 0 || page_size <= 0 || ldc < nh * dh) return IC_ERR_ARG;
+    if (!ic_gemm_qkv_rope_supported(IC_BF16, dh)) return IC_ERR_UNSUPPORTED;
+    if (((uintptr_t)cos_t & 15) || ((uintptr_t)sin_t & 15)) return IC_ERR_ARG;
+    const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
+    const RopeEpilogue rope{positions, slots, cos_t, sin_t, kcache, vcache, nh, nkvh, dh, page_size};
+    const int N = (nh + 2 * nkvh) * dh;
+    const int blocks = (nh + nkvh) * (dh / 32) + nkvh * (dh / 32);
+    dim3 grid(blocks, 1);
+#define IC_ROPE(WPB, UN, AL)                                                                             \
+    hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, WPB, UN, AL, 2>), grid, dim3(WPB * 64), 0, stream, \
+                       (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope)
+    if (blocks < 300) { if (aligned) IC_ROPE(16, 4, true); else IC_ROPE(16, 4, false); }
+    else { if (aligned) IC_ROPE(8, 4, true); else IC_ROPE(8, 4, false); }
+#undef IC_ROPE
     return ic_launch_status();
 }

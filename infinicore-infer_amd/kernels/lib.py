@@ -42,6 +42,8 @@ _SIGNATURES = {
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
     "ic_gemm_nt_supported": [_I, _I, _I],
+    "ic_gemm_qkv_rope_supported": [_I, _I],
+    "ic_gemm_qkv_rope": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
     "ic_gemm_nt_cfg": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
 }
 

@@ -262,3 +262,34 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False):
                                out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),
                                out.stride(0), float(alpha), 1 if swiglu_output else 0, _stream()), "gemm_nt")
     return out
+
+
+def gemm_qkv_rope_supported(dtype, head_dim: int) -> bool:
+    try:
+        return bool(get_lib().ic_gemm_qkv_rope_supported(dtype_code(dtype), head_dim))
+    except KernelError:
+        return False
+
+
+def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads, n_kv_heads, head_dim, page_size):
+    """For M <= 16 rows: qkv = a @ w^T with the rotary encoding and the cache write in the epilogue.
+    The q heads of qkv[M, >= n_heads * head_dim] hold rotated queries afterwards; rotated keys and
+    the values are in cache slot ``slots[m]``.  Full rotary, bfloat16."""
+    _dev(a, w, qkv, positions, slots, cos, sin, kcache, vcache)
+    M, K = a.shape
+    _i32(positions, "positions")
+    _i32(slots, "slots")
+    _need(M <= 16 and positions.numel() == M and slots.numel() == M, "gemm_qkv_rope: at most 16 rows, one position and slot each")
+    _need(tuple(w.shape) == ((n_heads + 2 * n_kv_heads) * head_dim, K), "gemm_qkv_rope: weight shape")
+    _need(qkv.shape[0] == M and qkv.shape[1] >= n_heads * head_dim and qkv.stride(1) == 1
+          and a.stride(1) == 1 and w.stride(1) == 1, "gemm_qkv_rope: layout")
+    _need(a.dtype == w.dtype == qkv.dtype == kcache.dtype == vcache.dtype == torch.bfloat16, "gemm_qkv_rope: bfloat16 only")
+    _need(cos.dtype == torch.float32 and sin.dtype == torch.float32 and cos.is_contiguous() and sin.is_contiguous()
+          and cos.shape[-1] == head_dim // 2 and sin.shape == cos.shape, "gemm_qkv_rope: cos/sin must be float32 [max_pos, dh/2]")
+    _need(kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape == vcache.shape
+          and tuple(kcache.shape[1:]) == (n_kv_heads, page_size, head_dim), "gemm_qkv_rope: cache layout")
+    check(get_lib().ic_gemm_qkv_rope(a.data_ptr(), w.data_ptr(), qkv.data_ptr(), M, K, a.stride(0), w.stride(0),
+                                     qkv.stride(0), positions.data_ptr(), slots.data_ptr(), cos.data_ptr(),
+                                     sin.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), n_heads, n_kv_heads,
+                                     head_dim, page_size, _stream()), "gemm_qkv_rope")
+    return qkv

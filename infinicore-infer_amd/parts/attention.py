@@ -76,8 +76,9 @@ class Attention(Mixer):
         nkv = 0 if (self.shared_kv or not cache.writes) else self.nkvh
         width = (self.nh + 2 * (0 if self.shared_kv else self.nkvh)) * self.dh
         qkv = ctx.ws.buffer("qkv", (T, width), rt.dtype)
-        linear(h, self.w_qkv, qkv, rt.gemm_impl)
-        self.pos_enc.rotate_and_store(qkv, ctx, cache, self.nh, nkv, self.dh)
+        if not self.pos_enc.project_rotate_store(h, self.w_qkv, qkv, ctx, cache, self.nh, nkv, self.dh):
+            linear(h, self.w_qkv, qkv, rt.gemm_impl)
+            self.pos_enc.rotate_and_store(qkv, ctx, cache, self.nh, nkv, self.dh)
         out = ctx.ws.buffer("attn_out", (T, self.nh * self.dh), rt.dtype)
         self._attend(qkv, out, ctx, cache)
         y = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)

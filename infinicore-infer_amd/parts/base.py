@@ -117,6 +117,11 @@ class PositionEncoding(Part):
         when n_kv_heads > 0, write k and v into ``cache`` at the step's slots."""
         raise NotImplementedError
 
+    def project_rotate_store(self, h, w_qkv, qkv, ctx, cache, n_heads: int, n_kv_heads: int, head_dim: int) -> bool:
+        """Optional shortcut: compute qkv = h w_qkv^T AND do what rotate_and_store does, in one
+        kernel.  Returns False (nothing done) when the part has no such kernel for this case."""
+        return False
+
 
 class Mixer(Part):
     category = "mixer"

@@ -69,6 +69,21 @@ class Rotary(PositionEncoding):
                           n_heads, n_kv_heads, head_dim, self.rot_dim, ctx.page_size)
 
 
+    def project_rotate_store(self, h, w_qkv, qkv, ctx, cache, n_heads, n_kv_heads, head_dim) -> bool:
+        """Few rows in bfloat16 with full rotary: the projection kernel rotates and writes the cache."""
+        from .linear import FEW_ROWS
+        rt = self.runtime
+        if (h.shape[0] > FEW_ROWS or rt.gemm_impl != "auto" or n_kv_heads == 0 or self.rot_dim != head_dim
+                or h.dtype != torch.bfloat16 or w_qkv.dtype != torch.bfloat16
+                or not ops.gemm_qkv_rope_supported(h.dtype, head_dim)):
+            return False
+        if ctx.max_position >= self.max_positions:
+            raise ValueError("position %d is beyond the rotary tables (%d)" % (ctx.max_position, self.max_positions))
+        ops.gemm_qkv_rope(h, w_qkv, qkv, ctx.positions, cache.slots, self.cos, self.sin, cache.k, cache.v,
+                          n_heads, n_kv_heads, head_dim, ctx.page_size)
+        return True
+
+
 @register_part("position_encoding", "none")
 class NoPositionEncoding(PositionEncoding):
     graph_safe = True

@@ -401,3 +401,35 @@ def test_gemm_nt_with_swiglu_output(cdtype, M, di, K):
     rnd = P.round_bf16 if cdtype == torch.bfloat16 else (lambda t: t)
     gu = rnd(P.plain_linear(h, w))
     _close(out, P.plain_swiglu(gu[:, :di], gu[:, di:]), cdtype, factor=2 if cdtype == torch.bfloat16 else 50)
+
+
+@pytest.mark.parametrize("M,nh,nkvh,dh,K,page", [(1, 4, 2, 32, 96, 16), (8, 6, 2, 64, 200, 16), (16, 3, 3, 64, 2304, 64),
+                                                 (5, 4, 1, 128, 344, 32), (3, 36, 36, 64, 2304, 64)])
+def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page):
+    """The fused projection + rotary + cache write equals the plain product followed by the
+    rotary/cache-write kernel."""
+    g = torch.Generator().manual_seed(31)
+    ops = _ops()
+    H = (nh + 2 * nkvh) * dh
+    h = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(H, K, generator=g) * 0.1).to(torch.bfloat16)
+    max_pos, n_pages = 300, 5
+    pos = torch.randint(0, max_pos, (M,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(n_pages * page, generator=g)[:M].to(torch.int32)
+    if M > 2:
+        slots[1] = -1                        # a row without a cache slot writes nothing
+    sin, cos = P.plain_rope_tables(dh, 10000.0, max_pos)
+    sin, cos = sin.float().to(DEV), cos.float().to(DEV)
+    kc = torch.zeros(n_pages, nkvh, page, dh, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    qkv = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_qkv_rope(h.to(DEV), w.to(DEV), qkv, pos.to(DEV), slots.to(DEV), cos, sin, kc, vc, nh, nkvh, dh, page)
+    # the two-kernel path
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ref = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_nt(h.to(DEV), w.to(DEV), ref)
+    ops.rope_kv_write(ref, pos.to(DEV), cos, sin, kc2, vc2, slots.to(DEV), nh, nkvh, dh, dh, page)
+    _close(qkv[:, :nh * dh], ref[:, :nh * dh], torch.bfloat16)
+    _close(kc, kc2, torch.bfloat16)
+    _close(vc, vc2, torch.bfloat16)
+    assert float(kc2.abs().max()) > 0 and float(vc2.abs().max()) > 0
