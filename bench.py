@@ -119,6 +119,7 @@ def main():
     ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
+    ap.add_argument("--no-tune", action="store_true", help="keep the library's default kernel choice for prefill products")
     ap.add_argument("--batch", type=int, default=BATCH, help="batch of the headline run (for profiling other points)")
     args = ap.parse_args()
     if args.gpus != 1:
@@ -134,7 +135,8 @@ def main():
     weight_bytes, kv_per_tok, prefill_flops = model_numbers(conf)
     vocab = conf.vocab_size
 
-    engine.tune_library_products([PROMPT])          # the library's kernel choice for 2,048-row products
+    if not args.no_tune:
+        engine.tune_library_products([PROMPT])      # the library's kernel choice for 2,048-row products
     g = torch.Generator().manual_seed(123)
     ptoks = torch.randint(0, vocab, (PROMPT,), generator=g).tolist()
     t_pf = time_prefill(engine, ptoks)
@@ -159,7 +161,7 @@ def main():
             "head_dim": conf.head_dim, "intermediate": conf.intermediate_size, "vocab": conf.vocab_size,
             "global_batch": BATCH, "seq_len": PROMPT, "context_mean": round(ctx, 1), "generated": args.steps,
             "page_size": args.page_size, "tied_embeddings": True, "parallelism": "single-gpu",
-            "sampling": "greedy on device", "library_gemm": "tuned for prefill",
+            "sampling": "greedy on device", "library_gemm": "default" if args.no_tune else "tuned for prefill",
         },
         "prefill": {"value": round(PROMPT / t_pf, 1), "tokens": PROMPT, "ms": round(t_pf * 1e3, 3),
                     "frac": round(pf_flops / t_pf / (PEAK_TFLOPS["bf16"] * 1e12), 4)},

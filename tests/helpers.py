@@ -41,13 +41,22 @@ TINY_C = dict(
                       long_factor=[1.0 + 0.09 * i for i in range(32)]))
 TINY_C_INIT = dict(std=0.05, norm_std=0.1)
 
-CONFIGS = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT)}
+# Tiny D: head size 128, four query heads on one kv head, hidden size below heads x head size.
+TINY_D = dict(
+    model_type="fm9g", vocab_size=300, hidden_size=136, num_hidden_layers=2, num_attention_heads=4,
+    num_key_value_heads=1, head_dim=128, intermediate_size=200, max_position_embeddings=384,
+    rms_norm_eps=1e-6, rope_theta=50000.0, scale_emb=2.0, dim_model_base=34, scale_depth=1.0,
+    tie_word_embeddings=True, eos_token_id=[])
+TINY_D_INIT = dict(std=0.06, norm_std=0.05)
+
+CONFIGS = {"A": (TINY_A, TINY_A_INIT), "B": (TINY_B, TINY_B_INIT), "C": (TINY_C, TINY_C_INIT),
+           "D": (TINY_D, TINY_D_INIT)}
 
 
 def make_model_dir(tmp_path, name, seed=0, dtype=torch.bfloat16):
     from infinicore_infer_amd.weights import write_random_model
     cfg, init = CONFIGS[name]
-    folder = os.path.join(str(tmp_path), "model_%s_%d" % (name, seed))
+    folder = os.path.join(str(tmp_path), "model_%s_%d_%s" % (name, seed, str(dtype).split(".")[-1]))
     if not os.path.isdir(folder):
         write_random_model(folder, cfg, seed=seed, dtype=dtype, **init)
     return folder

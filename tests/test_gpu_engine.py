@@ -10,7 +10,8 @@ import helpers as H
 pytestmark = pytest.mark.gpu
 
 DTYPES = [("float32", torch.float32, H.FP32_TOL), ("bfloat16", torch.bfloat16, H.BF16_TOL)]
-LENGTHS = {"A": [1, 7, 33, 100, 128, 45], "B": [5, 64, 130, 17, 256, 90], "C": [3, 150, 65, 300, 129, 40]}
+LENGTHS = {"A": [1, 7, 33, 100, 128, 45], "B": [5, 64, 130, 17, 256, 90], "C": [3, 150, 65, 300, 129, 40],
+           "D": [2, 200, 31, 384, 64, 129]}
 
 
 def _requests(name, seed=0):
@@ -50,7 +51,7 @@ MODES = {
 
 @pytest.mark.parametrize("mode", list(MODES))
 @pytest.mark.parametrize("dname,dtype,tol", DTYPES)
-@pytest.mark.parametrize("name", ["A", "B", "C"])
+@pytest.mark.parametrize("name", ["A", "B", "C", "D"])
 def test_replay_modes(tmp_path_factory, name, dname, dtype, tol, mode):
     requests = _requests(name)
     steps, max_tokens = MODES[mode](requests)
@@ -193,3 +194,17 @@ def test_trace_run_program(tmp_path):
                     i += 1
                 cursor[e["id"]] = cursor.get(e["id"], 0) + len(e["tokens"])
         H.compare(got, ref, tol, "trace_run " + dname)
+
+
+def test_weights_stored_in_32_bit_stay_so_in_bfloat16_mode(tmp_path_factory):
+    """A folder whose tensors are all float32, run with --dtype bfloat16: matrices stay float32
+    (their products run in float32), activations and the cache are bfloat16."""
+    from infinicore_infer_amd.engine import Engine
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "B", seed=4, dtype=torch.float32)
+    requests = {"a": H.random_tokens(509, 70, 1), "b": H.random_tokens(509, 33, 2)}
+    steps, max_tokens = H.trace_mixed(requests, sizes=(11, 2, 6), tail=4)
+    engine = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=max_tokens, page_size=16, max_requests=4)
+    assert engine.model.layers[0].mixer.w_qkv.dtype == torch.float32
+    assert engine.storage.kv(0)[0].dtype == torch.bfloat16
+    ref = H.plain_logits(H.CONFIGS["B"][0], H.load_state_dict(folder), requests, True)
+    H.compare(H.run_trace(engine, steps), ref, H.BF16_TOL, "float32 folder in bfloat16 mode")
