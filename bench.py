@@ -26,6 +26,18 @@ MODEL = dict(
     num_attention_heads=36, num_key_value_heads=36, intermediate_size=5760,
     max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0,
     scale_emb=12, dim_model_base=256, scale_depth=1.4, tie_word_embeddings=True, eos_token_id=2)
+# Other shapes of BASELINE.json (configs[3], configs[4]), for --shape; the default run is configs[2].
+SHAPES = {
+    "2b": MODEL,
+    "1b": dict(MODEL, vocab_size=73440, hidden_size=1536, num_hidden_layers=52, num_attention_heads=24,
+               num_key_value_heads=8, intermediate_size=3840),
+    "8b": dict(MODEL, vocab_size=73448, hidden_size=4096, num_hidden_layers=32, num_attention_heads=32,
+               num_key_value_heads=2, intermediate_size=16384, rms_norm_eps=1e-6, tie_word_embeddings=False,
+               max_position_embeddings=32768,
+               rope_scaling=dict(type="longrope", original_max_position_embeddings=32768,
+                                 short_factor=[1.0 + 3.0 * i / 63 for i in range(64)],
+                                 long_factor=[1.0 + 3.0 * i / 63 for i in range(64)])),
+}
 PROMPT = 2048
 BATCH = 8
 WEIGHT_STD = 0.1
@@ -40,10 +52,10 @@ def build_engine(layers, max_tokens, max_requests, page_size):
     from infinicore_infer_amd.engine import Engine
     from infinicore_infer_amd.parts import Runtime, build_model
     from infinicore_infer_amd.weights import init_random_weights
-    cfg = dict(MODEL, num_hidden_layers=layers)
+    cfg = dict(MODEL, num_hidden_layers=layers or MODEL["num_hidden_layers"])
     conf = config_from_dict(cfg)
     model = build_model(conf.model_spec(), Runtime(dtype=torch.bfloat16, device="cuda:0"))
-    init_random_weights(model, seed=0, std=WEIGHT_STD, tie=True)
+    init_random_weights(model, seed=0, std=WEIGHT_STD, tie=bool(cfg.get("tie_word_embeddings", True)))
     return Engine(model, max_tokens=max_tokens, page_size=page_size, max_requests=max_requests), conf
 
 
@@ -52,7 +64,7 @@ def model_numbers(conf):
     d, L, di, V = conf.hidden_size, conf.num_hidden_layers, conf.intermediate_size, conf.vocab_size
     nh, nkvh, dh = conf.num_attention_heads, conf.num_key_value_heads, conf.head_dim
     per_layer = (nh + 2 * nkvh) * dh * d + nh * dh * d + 3 * d * di
-    weight_bytes = 2 * (L * per_layer + V * d) + 4 * d * (2 * L + 1)
+    weight_bytes = 2 * (L * per_layer + V * d) + 4 * d * (2 * L + 1)      # the head's table once; embedding rows are negligible
     kv_bytes_per_token = 2 * L * nkvh * dh * 2
 
     def prefill_flops(T):
@@ -111,12 +123,14 @@ def time_decode(engine, batch, steps, warmup, vocab, seed=0):
 
 
 def main():
-    global BATCH
+    global BATCH, MODEL, PROMPT
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
-    ap.add_argument("--layers", type=int, default=MODEL["num_hidden_layers"])
+    ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
+    ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="2b is the benchmark's configuration")
+    ap.add_argument("--prompt", type=int, default=PROMPT)
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's default kernel choice for prefill products")
@@ -127,6 +141,7 @@ def main():
         return 2
 
     sys.path.insert(0, __import__("os").path.dirname(__import__("os").path.abspath(__file__)))
+    MODEL, PROMPT = SHAPES[args.shape], args.prompt
     per_req = PROMPT + args.warmup + args.steps + 64
     per_req = (per_req + 63) // 64 * 64
     BATCH = args.batch
@@ -151,16 +166,16 @@ def main():
     achieved = bytes_step / results[BATCH][0] / 1e9
 
     out = {
-        "metric": "decode tokens/s, batch %d, 2048-token prompts (MiniCPM-2B-shaped)" % BATCH,
+        "metric": "decode tokens/s, batch %d, %d-token prompts (MiniCPM-%s-shaped)" % (BATCH, PROMPT, args.shape.upper()),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
         "dtype": "bf16", "data": "synthetic (seeded random weights N(0,0.1) and token ids)",
         "config": {
-            "model": "MiniCPM-2B-shaped", "layers": conf.num_hidden_layers, "layers_of_config": MODEL["num_hidden_layers"],
+            "model": "MiniCPM-%s-shaped" % args.shape.upper(), "layers": conf.num_hidden_layers, "layers_of_config": MODEL["num_hidden_layers"],
             "hidden": conf.hidden_size, "heads": conf.num_attention_heads, "kv_heads": conf.num_key_value_heads,
             "head_dim": conf.head_dim, "intermediate": conf.intermediate_size, "vocab": conf.vocab_size,
             "global_batch": BATCH, "seq_len": PROMPT, "context_mean": round(ctx, 1), "generated": args.steps,
-            "page_size": args.page_size, "tied_embeddings": True, "parallelism": "single-gpu",
+            "page_size": args.page_size, "tied_embeddings": bool(MODEL.get("tie_word_embeddings", True)), "parallelism": "single-gpu",
             "sampling": "greedy on device", "library_gemm": "default" if args.no_tune else "tuned for prefill",
         },
         "prefill": {"value": round(PROMPT / t_pf, 1), "tokens": PROMPT, "ms": round(t_pf * 1e3, 3),

@@ -10,6 +10,7 @@ portions of prompts and single decoded tokens may be mixed and cut anywhere.
 from dataclasses import dataclass, field
 from typing import Dict, List, Optional, Sequence
 
+import numpy as np
 import torch
 
 from ..cache import CacheManager, CacheStorage, GroupSpec, OutOfPages
@@ -165,9 +166,9 @@ class Engine:
             seen.add(e.req_id)
             if len(e.tokens) == 0:
                 raise ValueError("request %r brings no tokens" % (e.req_id,))
-            for t in e.tokens:
-                if not (0 <= int(t) < vocab):
-                    raise ValueError("token id %r of request %r is outside the vocabulary (%d)" % (t, e.req_id, vocab))
+            if min(e.tokens) < 0 or max(e.tokens) >= vocab:
+                raise ValueError("a token id of request %r is outside the vocabulary (%d): %r"
+                                 % (e.req_id, vocab, [t for t in e.tokens if not 0 <= t < vocab][:5]))
             for w in e.want:
                 if not (0 <= int(w) < len(e.tokens)):
                     raise ValueError("wanted place %r of request %r is outside its %d tokens" % (w, e.req_id, len(e.tokens)))
@@ -205,17 +206,15 @@ class Engine:
     def _build_context(self, entries, starts) -> StepContext:
         ps = self.page_size
         R = len(entries)
-        T = sum(len(e.tokens) for e in entries)
-        tokens, positions, token_req, want_rows = [], [], [], []
-        decode_rows, tiles = [], []
+        lens = [len(e.tokens) for e in entries]
+        T = sum(lens)
         req_start = [0]
+        for n in lens:
+            req_start.append(req_start[-1] + n)
+        want_rows, decode_rows, tiles = [], [], []
         max_ctx = 0
-        for r, (e, p0) in enumerate(zip(entries, starts)):
-            n = len(e.tokens)
-            row0 = req_start[-1]
-            tokens.extend(int(t) for t in e.tokens)
-            positions.extend(range(p0, p0 + n))
-            token_req.extend([r] * n)
+        for r, (e, p0, n) in enumerate(zip(entries, starts, lens)):
+            row0 = req_start[r]
             want_rows.extend(row0 + int(w) for w in e.want)
             if n == 1:
                 decode_rows.append(row0)
@@ -223,46 +222,49 @@ class Engine:
             else:
                 for o in range(0, n, self._tile_rows):
                     tiles.append((r, row0 + o, min(self._tile_rows, n - o), p0 + o))
-            req_start.append(row0 + n)
         state_slots = [self.cache.state_slot(e.req_id) for e in entries]
         # tiles that see the most keys go first, so the longest blocks do not form the tail
         tiles.sort(key=lambda t: -(t[3] + t[2]))
-        tiles = [v for t in tiles for v in t]
 
-        group_slots, group_tables, group_maxb = [], [], []
-        for g in range(len(self.groups)):
-            sl = []
-            maxb = 1
-            for e, p0 in zip(entries, starts):
-                table = self.cache.block_table(e.req_id, g)
-                maxb = max(maxb, len(table))
-                for p in range(p0, p0 + len(e.tokens)):
-                    sl.append(table[p // ps] * ps + p % ps)
-            bt = []
-            for e in entries:
-                table = self.cache.block_table(e.req_id, g)
-                bt.extend(max(p, 0) for p in table)      # pages given back are never read; keep the index valid
-                bt.extend([0] * (maxb - len(table)))
-            group_slots.append(sl)
-            group_tables.append(bt)
-            group_maxb.append(maxb)
-
-        sections = [("tokens", tokens), ("positions", positions), ("token_req", token_req),
-                    ("state_slots", state_slots), ("want_rows", want_rows), ("decode_rows", decode_rows),
-                    ("tiles", tiles)]
-        for g in range(len(self.groups)):
-            sections.append(("slots%d" % g, group_slots[g]))
-            sections.append(("tables%d" % g, group_tables[g]))
+        n_groups = len(self.groups)
+        tables = [[self.cache.block_table(e.req_id, g) for e in entries] for g in range(n_groups)]
+        group_maxb = [max([1] + [len(t) for t in tables[g]]) for g in range(n_groups)]
+        sizes = [("tokens", T), ("positions", T), ("token_req", T), ("state_slots", R),
+                 ("want_rows", len(want_rows)), ("decode_rows", len(decode_rows)), ("tiles", 4 * len(tiles))]
+        for g in range(n_groups):
+            sizes += [("slots%d" % g, T), ("tables%d" % g, R * group_maxb[g])]
         offsets, total = {}, 0
-        for name, data in sections:
-            offsets[name] = (total, len(data))
-            total += _align4(len(data))
+        for name, n in sizes:
+            offsets[name] = (total, n)
+            total += _align4(n)
         host = self._ring.get(total)
-        flat: List[int] = []
-        for name, data in sections:
-            flat.extend(data)
-            flat.extend([0] * (_align4(len(data)) - len(data)))
-        host[:total] = torch.tensor(flat, dtype=torch.int32)
+        a = host.numpy()
+
+        def put(name, values):
+            o, n = offsets[name]
+            a[o:o + n] = values
+
+        for r, (e, p0, n) in enumerate(zip(entries, starts, lens)):     # per request, vectorised over its tokens
+            row0 = req_start[r]
+            o = offsets["tokens"][0] + row0
+            a[o:o + n] = e.tokens
+            o = offsets["positions"][0] + row0
+            pos = np.arange(p0, p0 + n, dtype=np.int32)
+            a[o:o + n] = pos
+            o = offsets["token_req"][0] + row0
+            a[o:o + n] = r
+            for g in range(n_groups):
+                table = np.asarray(tables[g][r], dtype=np.int32)
+                o = offsets["slots%d" % g][0] + row0
+                a[o:o + n] = table[pos // ps] * ps + pos % ps
+                o = offsets["tables%d" % g][0] + r * group_maxb[g]
+                a[o:o + len(table)] = np.maximum(table, 0)     # pages given back are never read; keep the index valid
+                a[o + len(table):o + group_maxb[g]] = 0
+        put("state_slots", state_slots)
+        put("want_rows", want_rows)
+        put("decode_rows", decode_rows)
+        if tiles:
+            put("tiles", np.asarray(tiles, dtype=np.int32).reshape(-1))
         if self._meta_dev is None or self._meta_dev.numel() < total:
             self._meta_dev = torch.empty(max(total, 4096), dtype=torch.int32, device=self.device)
         dev = self._meta_dev
@@ -281,12 +283,12 @@ class Engine:
         ctx.decode_rows, ctx.n_decode_rows = view("decode_rows"), len(decode_rows)
         ctx.decode_rows_identity = (len(decode_rows) == T)
         ctx.prefill_tiles = view("tiles").view(-1, 4)
-        ctx.n_prefill_tiles = len(tiles) // 4
+        ctx.n_prefill_tiles = len(tiles)
         ctx.req_start, ctx.req_pos = req_start, list(starts)
-        ctx.req_len = [len(e.tokens) for e in entries]
+        ctx.req_len = lens
         ctx.req_ids = [e.req_id for e in entries]
         ctx.host_state_slots = state_slots
-        ctx.max_position = max(positions)
+        ctx.max_position = max(p0 + n - 1 for p0, n in zip(starts, lens))
         ctx.max_context = _context_bucket(max_ctx) if max_ctx else 0
         ctx.cu_count = self.cu_count
         for slot in range(self.model.spec.num_cache_slots()):
