@@ -20,13 +20,14 @@ import torch
 HBM_PEAK_GBS = 8000.0           # MI355X HBM3E
 PEAK_TFLOPS = {"bf16": 2500.0, "fp32": 157.3}
 
-# BASELINE.json configs[2]: MiniCPM-2B-shaped
+# The benchmark's configuration: MiniCPM-2B-shaped (40 layers, hidden 2304, 36 heads of 64, vocabulary 122753)
 MODEL = dict(
     model_type="minicpm", vocab_size=122753, hidden_size=2304, num_hidden_layers=40,
     num_attention_heads=36, num_key_value_heads=36, intermediate_size=5760,
     max_position_embeddings=4096, rms_norm_eps=1e-5, rope_theta=10000.0,
     scale_emb=12, dim_model_base=256, scale_depth=1.4, tie_word_embeddings=True, eos_token_id=2)
-# Other shapes of BASELINE.json (configs[3], configs[4]), for --shape; the default run is configs[2].
+# Two further shapes for --shape: MiniCPM-1B-shaped (deep, narrow, 3 query heads per kv head) and
+# MiniCPM4-8B/FM9G-8B-shaped (16 query heads per kv head, head size 128, longrope).  The default run is 2b.
 SHAPES = {
     "2b": MODEL,
     "1b": dict(MODEL, vocab_size=73440, hidden_size=1536, num_hidden_layers=52, num_attention_heads=24,

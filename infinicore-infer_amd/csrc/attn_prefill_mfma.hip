@@ -36,7 +36,7 @@ union Frag8 {
 };
 
 template <int DH>
-__global__ void __launch_bounds__(kPfThreads)
+__global__ void __launch_bounds__(kPfThreads, (DH <= 64 ? 3 : 1))
 attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                          const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                          const int* __restrict__ block_tables, int bt_stride, const int4* __restrict__ tiles,
