@@ -12,6 +12,7 @@ ids.  One JSON line is printed.
 import argparse
 import json
 import math
+import os
 import sys
 import time
 
@@ -141,7 +142,7 @@ def main():
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
         return 2
 
-    sys.path.insert(0, __import__("os").path.dirname(__import__("os").path.abspath(__file__)))
+    sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
     MODEL, PROMPT = SHAPES[args.shape], args.prompt
     per_req = PROMPT + args.warmup + args.steps + 64
     per_req = (per_req + 63) // 64 * 64

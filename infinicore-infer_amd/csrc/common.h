@@ -4,6 +4,7 @@
 #pragma once
 #include <hip/hip_runtime.h>
 #include <hip/hip_bf16.h>
+#include "infinicore_infer_hip.h"
 #include <stdint.h>
 #include <math.h>
 

@@ -1,0 +1,64 @@
+// C interface of the gfx950 kernel library (libinfinicore_infer_hip-<hash>.so).
+//
+// Every function launches on `stream` and returns 0 when the launch was queued,
+// IC_ERR_ARG (-1) for a shape, stride, alignment or size the kernel does not take,
+// IC_ERR_UNSUPPORTED (-2) for a dtype or head size without a kernel, or the
+// (positive) hipError_t of a failed launch.  Nothing here allocates device memory;
+// scratch buffers are passed in by the caller.  dtype codes: 0 = float32, 1 = bfloat16.
+//
+// Cache layout of one layer: K and V planes [num_pages, n_kv_heads, page_size, head_dim].
+// Block tables: int32 [requests, bt_stride], logical page -> page id.
+#pragma once
+#include <hip/hip_runtime.h>
+
+#ifdef __cplusplus
+extern "C" {
+#endif
+
+// ---- elementwise.hip ---------------------------------------------------------------------
+// x[t, :] = table[tokens[t], :] * scale (x float32).
+int ic_embed(const int* tokens, const void* table, int table_dtype, float* x, int T, int d, float scale, hipStream_t stream);
+// out[r, :] = x[rows ? rows[r] : r, :] * rsqrt(mean(x^2) + eps) * w * out_scale (x, w float32).
+int ic_rmsnorm(const float* x, const int* rows, const float* w, void* out, int out_dtype, int n_rows, int d, float eps, float out_scale, hipStream_t stream);
+// x += alpha * y, then out = rmsnorm(x) * w.
+int ic_add_rmsnorm(float* x, const void* y, int y_dtype, float alpha, const float* w, void* out, int out_dtype, int T, int d, float eps, hipStream_t stream);
+// x += alpha * y over n elements.
+int ic_residual_add(float* x, const void* y, int y_dtype, float alpha, long long n, hipStream_t stream);
+// out[t, j] = up * silu(gate), gate = gate_up[t, j], up = gate_up[t, di + j].
+int ic_swiglu(const void* gate_up, void* out, int dtype, int T, int di, hipStream_t stream);
+
+// ---- rope_kv.hip ------------------------------------------------------------------------------
+// Rotary on the q and k heads of qkv[T, row_stride] (pairs (j, j + rot/2)), k and v written to cache slot slots[t].
+int ic_rope_kv_write(void* qkv, int dtype, const int* positions, const float* cos_t, const float* sin_t, void* kcache, void* vcache, const int* slots, int T, int row_stride, int nh, int nkvh, int dh, int rot, int page_size, hipStream_t stream);
+
+// ---- attention ------------------------------------------------------------------------------------
+// General kernel: any head size <= 512, float32 or bfloat16, optional window (0 = none).
+int ic_attn_generic(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* token_req, const int* positions, int T, int nh, int nkvh, int dh, int page_size, float scale, int window, hipStream_t stream);
+// Split-key kernel for single new tokens.  part_acc: float32 [n_tok, nh, nsplit, dh]; part_ml: float32 [n_tok, nh, nsplit, 2]; nsplit <= 64.
+int ic_attn_decode_supported(int dtype, int dh);
+int ic_attn_decode(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tok_list, const int* token_req, const int* positions, float* part_acc, float* part_ml, int n_tok, int nh, int nkvh, int dh, int page_size, float scale, int window, int nsplit, hipStream_t stream);
+// Matrix-core kernel for prompt portions.  tiles: int32 [n_tiles, 4] = (request row, first token row, rows <= tile_rows, first position).
+int ic_attn_prefill_supported(int dtype, int dh, int page_size);
+int ic_attn_prefill_tile_rows();
+int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, hipStream_t stream);
+
+// ---- gemm.hip ---------------------------------------------------------------------------------------
+// C[M, N] = alpha * A[M, K] W[N, K]^T, bfloat16 operands, float32 accumulation.  c_mode 1 (M <= 16):
+// W = [gate; up], C[M, N/2] = up * silu(gate).
+int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype);
+int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode, hipStream_t stream);
+// The same with the tiling chosen by the caller (tuning and tests); nt == 0 selects the SwiGLU variant.
+int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int nt, int wpb, int unroll, hipStream_t stream);
+// QKV projection of M <= 16 rows with rotary and cache write in the epilogue.
+int ic_gemm_qkv_rope_supported(int dtype, int dh);
+int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc, const int* positions, const int* slots, const float* cos_t, const float* sin_t, void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size, hipStream_t stream);
+
+// ---- sampling.hip -----------------------------------------------------------------------------------
+// Greedy choice per row; scratch_val / scratch_idx: 64 * n_rows elements.
+int ic_argmax(const float* logits, long long row_stride, int n_rows, int V, float* scratch_val, int* scratch_idx, int* out, hipStream_t stream);
+// Temperature / top-k / top-p with one uniform draw per row; temperature == nullptr: argmax.
+int ic_sample(const float* logits, long long row_stride, int n_rows, int V, const float* temperature, const int* top_k, const float* top_p, const float* uniform, int* out, hipStream_t stream);
+
+#ifdef __cplusplus
+}
+#endif

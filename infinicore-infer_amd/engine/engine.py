@@ -97,8 +97,6 @@ class Engine:
         self.groups: List[GroupSpec] = [
             GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots))
             for (nkv, dh, w), slots in keyed.items()]
-        if not self.groups:                  # a model without paged mixers still has a (tiny) page pool
-            self.groups = []
         self.cache = CacheManager(self.groups, [self.num_pages] * len(self.groups), self.page_size,
                                   self.max_requests, model.spec.max_positions)
         self.storage = CacheStorage(self.groups, [self.num_pages] * len(self.groups), self.page_size,
