@@ -160,7 +160,8 @@ def plain_swiglu(gate, up):
 # --------------------------------------------------------------------------
 # whole model                                  src/models/jiuge/jiuge.cpp:195-267
 # --------------------------------------------------------------------------
-def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", window=None, start_pos=0):
+def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", window=None, start_pos=0,
+                  rows=None):
     """Logits [T, vocab] (float64) of one request's whole token sequence from
     position 0.  ``weights``: tensors by checkpoint name (jiuge.py:33-77)."""
     rnd = rnd or _ident
@@ -198,6 +199,8 @@ def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", 
         up = rnd(plain_linear(h, weights[p + "mlp.up_proj.weight"]))
         act = rnd(plain_swiglu(gate, up))
         x = x + s_res * rnd(plain_linear(act, weights[p + "mlp.down_proj.weight"]))   # jiuge.cpp:249
+    if rows is not None:                       # only these positions' logits (the step function's choice, jiuge.cpp:270-277)
+        x = x[torch.as_tensor(rows, dtype=torch.long)]
     h = rnd(plain_rmsnorm(x, weights["model.norm.weight"], eps) * s_out)              # jiuge.py:198-201
     return plain_linear(h, head)                                                       # jiuge.cpp:264
 

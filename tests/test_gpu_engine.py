@@ -208,3 +208,44 @@ def test_weights_stored_in_32_bit_stay_so_in_bfloat16_mode(tmp_path_factory):
     assert engine.storage.kv(0)[0].dtype == torch.bfloat16
     ref = H.plain_logits(H.CONFIGS["B"][0], H.load_state_dict(folder), requests, True)
     H.compare(H.run_trace(engine, steps), ref, H.BF16_TOL, "float32 folder in bfloat16 mode")
+
+
+def test_benchmark_shaped_layers(tmp_path_factory):
+    """Two layers with the benchmark model's sizes (hidden 2304, 36 heads of 64, intermediate 5760,
+    an odd vocabulary of 30001), bfloat16: a prompt in portions that span several attention tiles, then
+    single tokens whose keys are split 16 ways, beside a second request; page size 64."""
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.weights import write_random_model
+    import os
+    cfg = dict(model_type="minicpm", vocab_size=30001, hidden_size=2304, num_hidden_layers=2,
+               num_attention_heads=36, num_key_value_heads=36, intermediate_size=5760,
+               max_position_embeddings=1024, rms_norm_eps=1e-5, rope_theta=10000.0, scale_emb=12,
+               dim_model_base=256, scale_depth=1.4, tie_word_embeddings=True, eos_token_id=2)
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "model_2b_shaped")
+    write_random_model(folder, cfg, seed=9, std=0.02)
+    sd = H.load_state_dict(folder)
+    a, b = H.random_tokens(30001, 420, 1), H.random_tokens(30001, 70, 2)
+    want_a, want_b = [0, 127, 128, 299, 300, 409] + list(range(410, 420)), [0, 69]
+    steps = [
+        {"step": 0, "entries": [{"id": "a", "tokens": a[:300], "want": [0, 127, 128, 299]}], "end": []},
+        {"step": 1, "entries": [{"id": "a", "tokens": a[300:410], "want": [0, 109]},
+                                {"id": "b", "tokens": b[:69], "want": [0]}], "end": []},
+    ]
+    for i in range(410, 420):
+        ents = [{"id": "a", "tokens": [a[i]], "want": [0]}]
+        if i == 410:
+            ents.append({"id": "b", "tokens": [b[69]], "want": [0]})
+        steps.append({"step": len(steps), "entries": ents, "end": ["b"] if i == 410 else []})
+    steps[-1]["end"] = ["a"]
+    engine = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=576, page_size=64, max_requests=2)
+    got = H.run_trace(engine, steps)
+    from plain_model import plain_forward, round_bf16
+    ref_a = plain_forward(cfg, sd, a, rnd=round_bf16, rows=want_a)
+    ref_b = plain_forward(cfg, sd, b, rnd=round_bf16, rows=want_b)
+    ref = {"a": {p: ref_a[i] for i, p in enumerate(want_a)}, "b": {p: ref_b[i] for i, p in enumerate(want_b)}}
+    assert sorted(got) == sorted([("a", p) for p in want_a] + [("b", p) for p in want_b])
+    scale = float(max(ref_a.abs().max(), ref_b.abs().max()))
+    for (rid, pos), row in got.items():
+        err = float((row.double() - ref[rid][pos]).abs().max()) / scale
+        assert err <= H.BF16_TOL, "request %s position %d differs by %.3g of the largest logit" % (rid, pos, err)
+    assert engine.graph_replays >= 9
