@@ -254,6 +254,224 @@ attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __res
     }
 }
 
+// ---------------------------------------------------------------------------------------------
+// Grouped queries on the matrix cores (bfloat16): the query heads that share a kv head are the
+// columns of one 16-wide tile, so keys and values are read once for the whole group.
+//
+// Same grid and partial-result layout as above.  A wave owns tiles of 32 keys of the block's
+// share (tile i -> wave i % 4).  S^T = K Q^T with v_mfma_f32_16x16x32_bf16, keys as rows: the K
+// operand comes straight from memory in operand layout (lane l: key l%16, dims 8(l/16)..+7 of a
+// 32-dim chunk).  A lane then holds 4+4 keys of ONE head (l%16), so the running softmax needs two
+// cross-lane steps.  O^T = V^T P^T: P^T is already the B operand (slot (l/16, e) stands for key
+// 4(l/16) + e of the first 16 keys for e < 4, of the second 16 for e >= 4); V goes through LDS
+// (written as rows, read as columns).  16x16x32 layout: A[i = l%16][k = 8(l/16)..+7],
+// B[k = 8(l/16)..+7][j = l%16], D[i = 4(l/16) + e][j = l%16].
+typedef __bf16 gq_bf16x8 __attribute__((ext_vector_type(8)));
+typedef float gq_v4f __attribute__((ext_vector_type(4)));
+typedef float gq_v8f __attribute__((ext_vector_type(8)));
+constexpr int kGqaKeys = 32;
+
+union GqFrag {
+    uint4 u;
+    uint16_t h[8];
+    gq_bf16x8 v;
+};
+
+template <int DH>
+__global__ void __launch_bounds__(kDecThreads)
+attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
+                       const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
+                       const int* __restrict__ block_tables, int bt_stride,
+                       const int* __restrict__ tok_list, const int* __restrict__ token_req,
+                       const int* __restrict__ positions,
+                       float* __restrict__ part_acc, float* __restrict__ part_ml,
+                       int nh, int nkvh, int page_size, float scale, int window, int nsplit) {
+    constexpr int NC = DH / 32;                    // 32-dim chunks of the score product
+    constexpr int ND = DH / 16;                    // 16-dim chunks of the output
+    constexpr int VS = DH + 8;                     // LDS row stride of a V tile (elements)
+    constexpr int NV = kGqaKeys * (DH / 8) / 64;   // 16-byte V loads per lane and tile
+    __shared__ __attribute__((aligned(16))) uint16_t Vs[kDecWaves][kGqaKeys * VS];
+    __shared__ float sm_ml[kDecWaves][16][2];
+    __shared__ int pages[kDecMaxPages];
+    static_assert(sizeof(uint16_t) * kGqaKeys * VS >= sizeof(float) * 16 * DH, "merge buffer fits in the V tiles");
+    float* sm_o = reinterpret_cast<float*>(&Vs[0][0]);       // [waves][16 heads][DH] after the key loop
+
+    const int split = blockIdx.x, kvh = blockIdx.y, n = blockIdx.z;
+    const int t = tok_list ? tok_list[n] : n;
+    const int g = nh / nkvh;
+    const int pos = positions[t];
+    const int* bt = block_tables + (size_t)token_req[t] * bt_stride;
+    const int lo0 = (window > 0 && pos - window + 1 > 0) ? pos - window + 1 : 0;
+    const int nkeys = pos + 1 - lo0;
+    const int per = (nkeys + nsplit - 1) / nsplit;
+    const int lo = lo0 + split * per;
+    int hi = lo + per;
+    if (hi > pos + 1) hi = pos + 1;
+
+    const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const int lr = lane & 15, lg = lane >> 4;      // row / column of a tile, and the lane group
+    const size_t head_stride = (size_t)page_size * DH;
+    const size_t page_stride = (size_t)nkvh * head_stride;
+    const uint16_t* kbase = kcache + (size_t)kvh * head_stride;
+    const uint16_t* vbase = vcache + (size_t)kvh * head_stride;
+
+    const int page_lo = lo / page_size;
+    const int n_pages = (hi > lo) ? (hi - 1) / page_size - page_lo + 1 : 0;
+    const bool staged = n_pages <= kDecMaxPages;
+    if (staged)
+        for (int i = threadIdx.x; i < n_pages; i += kDecThreads) pages[i] = bt[page_lo + i];
+    __syncthreads();
+    auto row_of = [&](int key) -> size_t {
+        const int lp = key / page_size;
+        const int pg = staged ? pages[lp - page_lo] : bt[lp];
+        return (size_t)pg * page_stride + (size_t)(key - lp * page_size) * DH;
+    };
+
+    const int n_tiles = (hi > lo) ? (hi - lo + kGqaKeys - 1) / kGqaKeys : 0;
+    const int rounds = (n_tiles + kDecWaves - 1) / kDecWaves;
+
+    for (int h0 = 0; h0 < g; h0 += 16) {
+        // Q^T operand: head lr of this chunk, dims 32c + 8 lg .. +7
+        GqFrag qf[NC];
+        {
+            const bool head_ok = h0 + lr < g;
+            const uint16_t* qp = q + (size_t)t * q_stride + (size_t)(kvh * g + h0 + (head_ok ? lr : 0)) * DH + 8 * lg;
+#pragma unroll
+            for (int c = 0; c < NC; ++c) {
+                if (head_ok) qf[c].u = *reinterpret_cast<const uint4*>(qp + 32 * c);
+                else qf[c].u = make_uint4(0, 0, 0, 0);
+            }
+        }
+        gq_v4f oacc[ND];
+#pragma unroll
+        for (int c = 0; c < ND; ++c) oacc[c] = gq_v4f{0.f, 0.f, 0.f, 0.f};
+        float m = -INFINITY, l = 0.f;              // of head lr, the same in the four lane groups
+
+        GqFrag kreg[2][NC];
+        uint4 vreg[NV];
+        auto fetch = [&](int tile) {
+            const int kt = lo + tile * kGqaKeys;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                const int key = kt + 16 * s2 + lr;
+                const bool ok = tile < n_tiles && key < hi;
+                const size_t off = ok ? row_of(key) + 8 * lg : 0;
+#pragma unroll
+                for (int c = 0; c < NC; ++c) {
+                    if (ok) kreg[s2][c].u = *reinterpret_cast<const uint4*>(kbase + off + 32 * c);
+                    else kreg[s2][c].u = make_uint4(0, 0, 0, 0);
+                }
+            }
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int idx = lane + 64 * i;
+                const int vkey = idx / (DH / 8), oct = idx - vkey * (DH / 8);
+                const int key = kt + vkey;
+                vreg[i] = make_uint4(0, 0, 0, 0);
+                if (tile < n_tiles && key < hi) vreg[i] = *reinterpret_cast<const uint4*>(vbase + row_of(key) + oct * 8);
+            }
+        };
+        auto stash = [&]() {
+#pragma unroll
+            for (int i = 0; i < NV; ++i) {
+                const int idx = lane + 64 * i;
+                const int vkey = idx / (DH / 8), oct = idx - vkey * (DH / 8);
+                *reinterpret_cast<uint4*>(&Vs[wave][vkey * VS + oct * 8]) = vreg[i];
+            }
+        };
+
+        // A wave writes and reads only its own V tile in LDS, and LDS serves a wave's instructions
+        // in order, so no block barrier is needed in this loop (wave_barrier keeps the compiler from
+        // moving LDS accesses across it).
+        fetch(wave);
+        for (int r = 0; r < rounds; ++r) {
+            const int tile = r * kDecWaves + wave;
+            if (tile >= n_tiles) break;             // uniform in the wave
+            const int kt = lo + tile * kGqaKeys;
+            __builtin_amdgcn_wave_barrier();
+            stash();
+            __builtin_amdgcn_wave_barrier();
+
+            // ---- S^T = K Q^T, two subtiles of 16 keys ----------------------------------
+            gq_v4f sacc[2];
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2) {
+                sacc[s2] = gq_v4f{0.f, 0.f, 0.f, 0.f};
+#pragma unroll
+                for (int c = 0; c < NC; ++c)
+                    sacc[s2] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(kreg[s2][c].v, qf[c].v, sacc[s2], 0, 0, 0);
+            }
+            fetch(tile + kDecWaves);                // the next tile's loads fly during the rest of this one
+            float sv[8];
+            float mloc = -INFINITY;
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    const int key = kt + 16 * s2 + 4 * lg + e;
+                    const float x = (key < hi) ? sacc[s2][e] * scale : -INFINITY;
+                    sv[4 * s2 + e] = x;
+                    mloc = fmaxf(mloc, x);
+                }
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
+            mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
+            const float m_new = fmaxf(m, mloc);     // finite: every tile has at least one key
+            const float corr = expf(m - m_new);
+            float rs = 0.f;
+            gq_v8f pf;
+#pragma unroll
+            for (int e = 0; e < 8; ++e) { const float p = expf(sv[e] - m_new); pf[e] = p; rs += p; }
+            rs += __shfl_xor(rs, 16, kWave);
+            rs += __shfl_xor(rs, 32, kWave);
+            l = l * corr + rs;
+            m = m_new;
+            const gq_bf16x8 pb = __builtin_convertvector(pf, gq_bf16x8);
+
+            // ---- O^T += V^T P^T ----------------------------------------------------------------
+            const uint16_t* vrow = &Vs[wave][(4 * lg) * VS + lr];
+#pragma unroll
+            for (int c = 0; c < ND; ++c) {
+                GqFrag a;
+#pragma unroll
+                for (int e = 0; e < 4; ++e) {
+                    a.h[e] = vrow[e * VS + 16 * c];
+                    a.h[4 + e] = vrow[(16 + e) * VS + 16 * c];
+                }
+                oacc[c] *= corr;
+                oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb, oacc[c], 0, 0, 0);
+            }
+        }
+
+        // ---- merge the four waves; O^T[d = 16c + 4 lg + e][head lr] ---------------------------
+        __syncthreads();
+#pragma unroll
+        for (int c = 0; c < ND; ++c)
+#pragma unroll
+            for (int e = 0; e < 4; ++e) sm_o[(wave * 16 + lr) * DH + 16 * c + 4 * lg + e] = oacc[c][e];
+        if (lg == 0) { sm_ml[wave][lr][0] = m; sm_ml[wave][lr][1] = l; }
+        __syncthreads();
+        for (int idx = threadIdx.x; idx < 16 * DH; idx += kDecThreads) {
+            const int j = idx / DH, d = idx - j * DH;
+            if (h0 + j >= g) continue;
+            float mm = -INFINITY;
+            for (int w = 0; w < kDecWaves; ++w) mm = fmaxf(mm, sm_ml[w][j][0]);
+            float a = 0.f, ll = 0.f;
+            if (mm != -INFINITY) {
+                for (int w = 0; w < kDecWaves; ++w) {
+                    const float cw = expf(sm_ml[w][j][0] - mm);
+                    a += sm_o[(w * 16 + j) * DH + d] * cw;
+                    ll += sm_ml[w][j][1] * cw;
+                }
+            }
+            const int h = kvh * g + h0 + j;
+            const size_t pidx = ((size_t)n * nh + h) * nsplit + split;
+            part_acc[pidx * DH + d] = a;
+            if (d == 0) { part_ml[pidx * 2] = mm; part_ml[pidx * 2 + 1] = ll; }
+        }
+        __syncthreads();                            // sm_o (the V tiles) is reused by the next chunk
+    }
+}
+
 template <typename T, int DH>
 static int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                          const void* vcache, const int* block_tables, int bt_stride, const int* tok_list,
@@ -261,7 +479,11 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
                          int n_tok, int nh, int nkvh, int page_size, float scale, int window, int nsplit,
                          hipStream_t stream) {
     dim3 grid(nsplit, nkvh, n_tok), block(kDecThreads);
-    if (nh == nkvh)
+    if (nh != nkvh && sizeof(T) == 2)
+        hipLaunchKernelGGL((attn_decode_gqa_kernel<DH>), grid, block, 0, stream, (const uint16_t*)q, q_stride,
+                           (const uint16_t*)kcache, (const uint16_t*)vcache, block_tables, bt_stride, tok_list,
+                           token_req, positions, part_acc, part_ml, nh, nkvh, page_size, scale, window, nsplit);
+    else if (nh == nkvh)
         hipLaunchKernelGGL((attn_decode_split_kernel<T, DH, 1>), grid, block, 0, stream, (const T*)q, q_stride,
                            (const T*)kcache, (const T*)vcache, block_tables, bt_stride, tok_list, token_req,
                            positions, part_acc, part_ml, nh, nkvh, page_size, scale, window, nsplit);

@@ -251,7 +251,7 @@ static void dispatch_gemm(const void* A, const void* W, void* C, int M, int N, i
 #define IC_GO(NT, MT, WPB, UN) launch_gemm<TC, NT, MT, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream)
     // tilings from a sweep over the projection shapes of 1B..8B models on MI355X
     if (M <= 16) {
-        if (tiles < 256) IC_GO(1, 1, 16, 2);
+        if (tiles < 400) IC_GO(1, 1, 16, 4);
         else if (tiles < 600) IC_GO(2, 1, 16, 4);
         else if (tiles < 2048) { if (M <= 4) IC_GO(1, 1, 8, 2); else IC_GO(1, 1, 4, 2); }
         else { if (M <= 8) IC_GO(1, 1, 16, 2); else IC_GO(4, 1, 4, 2); }
