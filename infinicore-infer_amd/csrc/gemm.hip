@@ -47,13 +47,33 @@ struct RopeEpilogue {
     int nh, nkvh, dh, page_size;
 };
 
+// A norm split over two products (M <= 16).  The product BEFORE the norm (EPI == 3) owns the
+// residual add: h = x + rscale * (its result), written back to x; it stores y = h * g (g: the
+// norm's weight) instead of its result, and per column block the sums of h^2 of every row.  The
+// product AFTER the norm takes y as its operand and multiplies row m of its result by
+// rsqrt(sum over the column blocks / width + eps): the norm's row factor commutes with the product.
+constexpr int kMaxSumParts = 256;
+struct NormFuse {
+    const float* ss_in;        // [n_parts_in, 16] sums of squares per column block and row; nullptr: rows are normed already
+    int n_parts_in;            // <= kMaxSumParts
+    float inv_width, eps;
+    float* x;                  // EPI == 3: float32 residual stream [M, N], row stride ldx, updated in place
+    int ldx;
+    const float* g;            // [N]
+    float rscale;
+    float* ss_out;             // [gridDim.x, 16]
+};
+
 template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI>
 __global__ void __launch_bounds__(WPB * 64)
 gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C,
-                    int M, int N, int K, int lda, int ldw, int ldc, float alpha, RopeEpilogue rope) {
+                    int M, int N, int K, int lda, int ldw, int ldc, float alpha, RopeEpilogue rope, NormFuse nf) {
     constexpr bool CSWIGLU = (EPI == 1);
     constexpr bool CROPE = (EPI == 2);
+    constexpr bool CRESID = (EPI == 3);
+    constexpr int PV = kMaxSumParts / (WPB * 4);             // column-block sums a thread fetches
     __shared__ float red[WPB - 1][NT * MT][64][4];
+    __shared__ float ssum[WPB * 4][16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
     // CSWIGLU: W = [gate rows (N/2); up rows (N/2)]; a block owns 16 gate rows and the matching
@@ -99,6 +119,26 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) acc[nt][mt] = v4f{0.f, 0.f, 0.f, 0.f};
 
+    // the row factors' partial sums are fetched first and used last: their latency hides behind the loop
+    float pv[PV];
+    if (nf.ss_in) {
+#pragma unroll
+        for (int i = 0; i < PV; ++i) {
+            const int b = (tid >> 4) + i * (WPB * 4);
+            pv[i] = (b < nf.n_parts_in) ? nf.ss_in[b * 16 + (tid & 15)] : 0.f;
+        }
+    }
+
+    // the residual epilogue's operands are fetched first as well
+    float xres[4] = {0.f, 0.f, 0.f, 0.f}, gres[4] = {0.f, 0.f, 0.f, 0.f};
+    if (CRESID && wave == 0 && m0 + r < M) {
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            const int n = n0 + 4 * kq + e;
+            if (n < N) { xres[e] = nf.x[(size_t)(m0 + r) * nf.ldx + n]; gres[e] = nf.g[n]; }
+        }
+    }
+
     // k-steps of 32 are dealt to the waves in turn; UNROLL steps are loaded before any is used
     const int nsteps = (K + 31) >> 5;
     for (int s0 = wave; s0 < nsteps; s0 += WPB * UNROLL) {
@@ -141,8 +181,24 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
                 for (int e = 0; e < 4; ++e) red[wave - 1][nt * MT + mt][lane][e] = acc[nt][mt][e];
     }
+    if (nf.ss_in) {
+        float t = 0.f;
+#pragma unroll
+        for (int i = 0; i < PV; ++i) t += pv[i];
+        ssum[tid >> 4][tid & 15] = t;
+    }
     __syncthreads();
     if (wave > 0) return;
+    float rowf = 1.0f;                                       // norm factor of row r (lanes of one column of D)
+    if (nf.ss_in) {
+        float t = 0.f;
+#pragma unroll
+        for (int j = 0; j < WPB; ++j) t += ssum[4 * j + kq][r];
+        t += __shfl_xor(t, 16, kWave);
+        t += __shfl_xor(t, 32, kWave);
+        rowf = rsqrtf(t * nf.inv_width + nf.eps);
+    }
+    alpha *= rowf;
     if (CSWIGLU) {
 #pragma unroll
         for (int mt = 0; mt < MT; ++mt) {
@@ -170,8 +226,8 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
             float a0 = acc[0][0][e], a1 = acc[NT - 1][0][e];
 #pragma unroll
             for (int w = 0; w < WPB - 1; ++w) { a0 += red[w][0][lane][e]; a1 += red[w][NT - 1][lane][e]; }
-            v0[e] = to_f32(from_f32<TC>(a0));           // the projection is rounded to its type first, as when stored
-            v1[e] = to_f32(from_f32<TC>(a1));
+            v0[e] = to_f32(from_f32<TC>(alpha * a0));   // the projection is rounded to its type first, as when stored
+            v1[e] = to_f32(from_f32<TC>(alpha * a1));
         }
         const int half = rope.dh >> 1;
         const int slot = rope.slots[m];
@@ -201,6 +257,28 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         }
         return;
     }
+    if (CRESID) {                                       // NT == MT == 1
+        const int m = m0 + r;
+        float ss = 0.f;
+#pragma unroll
+        for (int e = 0; e < 4; ++e) {
+            float v = acc[0][0][e];
+#pragma unroll
+            for (int w = 0; w < WPB - 1; ++w) v += red[w][0][lane][e];
+            const int n = n0 + 4 * kq + e;
+            if (m < M && n < N) {
+                const float d = to_f32(from_f32<TC>(alpha * v));     // the branch's output as it would be stored
+                const float h = xres[e] + nf.rscale * d;
+                nf.x[(size_t)m * nf.ldx + n] = h;
+                C[(size_t)m * ldc + n] = from_f32<TC>(h * gres[e]);
+                ss += h * h;
+            }
+        }
+        ss += __shfl_xor(ss, 16, kWave);
+        ss += __shfl_xor(ss, 32, kWave);
+        if (kq == 0) nf.ss_out[blockIdx.x * 16 + r] = ss;
+        return;
+    }
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
@@ -217,38 +295,38 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         }
 }
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL>
+template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0>
 static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
-                        int ldc, float alpha, bool aligned, hipStream_t stream) {
+                        int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream) {
     dim3 grid((N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, 0>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{});
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, 0>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{});
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, EPI>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
 }
 
 // The gate/up projection with the activation in its epilogue: W [N, K] = [gate; up], C [M, N/2].
 template <typename TC, int WPB, int UN = 2>
 static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
-                               int ldc, bool aligned, hipStream_t stream) {
+                               int ldc, bool aligned, const NormFuse& nf, hipStream_t stream) {
     dim3 grid((N / 2 + 15) / 16, (M + 15) / 16), block(WPB * 64);
     if (aligned)
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, true, 1>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{});
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
     else
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, false, 1>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{});
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
 }
 
 // NT weight tiles of 16 rows share one load of the A fragments; WPB waves split K.  Both are
 // chosen so that (column blocks x waves) fills the chip's SIMDs about twice over.
 template <typename TC>
 static void dispatch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
-                          int ldc, float alpha, bool aligned, hipStream_t stream) {
+                          int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream) {
     const int tiles = (N + 15) / 16;
-#define IC_GO(NT, MT, WPB, UN) launch_gemm<TC, NT, MT, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream)
+#define IC_GO(NT, MT, WPB, UN) launch_gemm<TC, NT, MT, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream)
     // tilings from a sweep over the projection shapes of 1B..8B models on MI355X
     if (M <= 16) {
         if (tiles < 400) IC_GO(1, 1, 16, 4);
@@ -270,11 +348,11 @@ static void dispatch_gemm(const void* A, const void* W, void* C, int M, int N, i
 template <typename TC, int NT, int WPB, int UN>
 static int launch_cfg_m(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                         float alpha, bool aligned, hipStream_t stream) {
-    if (M <= 16) launch_gemm<TC, NT, 1, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
-    else if (M <= 32) launch_gemm<TC, NT, 2, WPB, (UN > 2 ? 2 : UN)>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
+    if (M <= 16) launch_gemm<TC, NT, 1, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, NormFuse{}, stream);
+    else if (M <= 32) launch_gemm<TC, NT, 2, WPB, (UN > 2 ? 2 : UN)>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, NormFuse{}, stream);
     else {
         if (NT * WPB > 32) return IC_ERR_UNSUPPORTED;       // would not fit LDS
-        launch_gemm<TC, (NT > 2 ? 2 : NT), 4, (WPB > 8 ? 8 : WPB), 1>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
+        launch_gemm<TC, (NT > 2 ? 2 : NT), 4, (WPB > 8 ? 8 : WPB), 1>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, NormFuse{}, stream);
     }
     return IC_OK;
 }
@@ -286,7 +364,7 @@ IC_EXPORT int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype,
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
     if (nt == 0) {                                  // nt == 0: the variant with SwiGLU in the epilogue
         if (M > 16 || (N & 1) || ldc < N / 2) return IC_ERR_ARG;
-#define IC_SW(WPB, UN) if (wpb == WPB && unroll == UN) { launch_gemm_swiglu<bf16, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream); return ic_launch_status(); }
+#define IC_SW(WPB, UN) if (wpb == WPB && unroll == UN) { launch_gemm_swiglu<bf16, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, aligned, NormFuse{}, stream); return ic_launch_status(); }
         IC_SW(4, 2) IC_SW(4, 4) IC_SW(8, 2) IC_SW(8, 4) IC_SW(16, 2) IC_SW(16, 4)
 #undef IC_SW
         return IC_ERR_UNSUPPORTED;
@@ -307,30 +385,60 @@ IC_EXPORT int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype) {
     return a_dtype == IC_BF16 && w_dtype == IC_BF16 && (c_dtype == IC_F32 || c_dtype == IC_BF16);
 }
 
+// Fills the kernel's description of a split norm from the C structs; false: an argument fault.
+static bool norm_fuse_args(const IcRowFactor* rf, const IcResidualNorm* tail, int M, int N, int K, int c_dtype,
+                           int col_blocks, NormFuse& nf) {
+    if (rf) {
+        if (M > 16 || !rf->sumsq || rf->n_parts <= 0 || rf->n_parts > kMaxSumParts || rf->width <= 0) return false;
+        nf.ss_in = rf->sumsq; nf.n_parts_in = rf->n_parts; nf.inv_width = 1.0f / (float)rf->width; nf.eps = rf->eps;
+    }
+    if (tail) {
+        if (M > 16 || c_dtype != IC_BF16 || !tail->x || !tail->weight || !tail->sumsq_out || tail->ldx < N ||
+            tail->n_parts != col_blocks || col_blocks > kMaxSumParts) return false;
+        nf.x = tail->x; nf.ldx = tail->ldx; nf.g = tail->weight; nf.rscale = tail->alpha; nf.ss_out = tail->sumsq_out;
+    }
+    return true;
+}
+
+// Column blocks (= sums of squares per row) that c_mode 2 writes for an N wide product.
+IC_EXPORT int ic_gemm_nt_residual_parts(int N) { return (N + 15) / 16; }
+
 // c_mode 0: C [M, N] = alpha * A W^T.  c_mode 1 (M <= 16, N even, alpha ignored): W = [gate; up] and
 // C [M, N/2] = up * silu(gate), both projections rounded to C's type before the activation.
+// c_mode 2 (M <= 16, bfloat16 C, `tail` given): x += tail->alpha * (alpha * A W^T); C = x * tail->weight;
+// tail->sumsq_out[b * 16 + m] = sum of x[m]^2 over column block b.  row_factor (M <= 16, any c_mode): row m
+// of the product is multiplied by rsqrt(sum_b sumsq[b * 16 + m] / width + eps) first.
 IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype,
                          int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode,
-                         hipStream_t stream) {
+                         const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream) {
     if (M <= 0 || N <= 0) return IC_OK;
-    if (K <= 0 || lda < K || ldw < K || c_mode < 0 || c_mode > 1) return IC_ERR_ARG;
+    if (K <= 0 || lda < K || ldw < K || c_mode < 0 || c_mode > 2) return IC_ERR_ARG;
     if (c_mode == 1 ? (M > 16 || (N & 1) || ldc < N / 2) : (ldc < N)) return IC_ERR_ARG;
+    if ((c_mode == 2) != (tail != nullptr)) return IC_ERR_ARG;
     if (!ic_gemm_nt_supported(a_dtype, w_dtype, c_dtype)) return IC_ERR_UNSUPPORTED;
     if ((M + 63) / 64 > 65535) return IC_ERR_ARG;
+    NormFuse nf{};
+    if (!norm_fuse_args(row_factor, tail, M, N, K, c_dtype, ic_gemm_nt_residual_parts(N), nf)) return IC_ERR_ARG;
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
+    if (c_mode == 2) {
+        // a long K over few columns (the down projection) does better with fewer, longer waves (from a sweep)
+        if (K > 2 * N) launch_gemm<bf16, 1, 1, 8, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream);
+        else launch_gemm<bf16, 1, 1, 16, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream);
+        return ic_launch_status();
+    }
     if (c_mode == 1) {
         const int tiles = (N / 2 + 15) / 16;
         if (c_dtype == IC_F32) {
-            if (tiles < 300) launch_gemm_swiglu<float, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
-            else launch_gemm_swiglu<float, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
+            if (tiles < 300) launch_gemm_swiglu<float, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
+            else launch_gemm_swiglu<float, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
         } else {
-            if (tiles < 300) launch_gemm_swiglu<bf16, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
-            else launch_gemm_swiglu<bf16, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, stream);
+            if (tiles < 300) launch_gemm_swiglu<bf16, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
+            else launch_gemm_swiglu<bf16, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
         }
         return ic_launch_status();
     }
-    if (c_dtype == IC_F32) dispatch_gemm<float>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
-    else dispatch_gemm<bf16>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, stream);
+    if (c_dtype == IC_F32) dispatch_gemm<float>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream);
+    else dispatch_gemm<bf16>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream);
     return ic_launch_status();
 }
 
@@ -343,7 +451,7 @@ IC_EXPORT int ic_gemm_qkv_rope_supported(int dtype, int dh) { return dtype == IC
 IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc,
                                const int* positions, const int* slots, const float* cos_t, const float* sin_t,
                                void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size,
-                               hipStream_t stream) {
+                               const IcRowFactor* row_factor, hipStream_t stream) {
     if (M <= 0) return IC_OK;
     if (M > 16 || K <= 0 || lda < K || ldw < K || nh <= 0 || nkvh <= 0 || page_size <= 0 || ldc < nh * dh) return IC_ERR_ARG;
     if (!ic_gemm_qkv_rope_supported(IC_BF16, dh)) return IC_ERR_UNSUPPORTED;
@@ -351,11 +459,13 @@ IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
     const RopeEpilogue rope{positions, slots, cos_t, sin_t, kcache, vcache, nh, nkvh, dh, page_size};
     const int N = (nh + 2 * nkvh) * dh;
+    NormFuse nf{};
+    if (!norm_fuse_args(row_factor, nullptr, M, N, K, IC_BF16, 0, nf)) return IC_ERR_ARG;
     const int blocks = (nh + nkvh) * (dh / 32) + nkvh * (dh / 32);
     dim3 grid(blocks, 1);
 #define IC_ROPE(WPB, UN, AL)                                                                             \
     hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, WPB, UN, AL, 2>), grid, dim3(WPB * 64), 0, stream, \
-                       (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope)
+                       (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf)
     if (blocks < 300) { if (aligned) IC_ROPE(16, 4, true); else IC_ROPE(16, 4, false); }
     else { if (aligned) IC_ROPE(8, 4, true); else IC_ROPE(8, 4, false); }
 #undef IC_ROPE

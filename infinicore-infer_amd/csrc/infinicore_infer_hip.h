@@ -43,15 +43,35 @@ int ic_attn_prefill_tile_rows();
 int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, hipStream_t stream);
 
 // ---- gemm.hip ---------------------------------------------------------------------------------------
+// A norm y = x * rsqrt(mean(x^2) + eps) * w between two products of M <= 16 rows can be split over them: the
+// product before it adds its result to the residual stream, stores x * w and the sums of x^2 per row and
+// column block (IcResidualNorm); the product after it multiplies each row of its result by the row's
+// rsqrt(sum / width + eps) (IcRowFactor).
+typedef struct {
+    const float* sumsq;   // [n_parts, 16]: sum of squares of row m over column block b at [b * 16 + m]
+    int n_parts;          // <= 256
+    int width;            // elements per row the sums run over
+    float eps;
+} IcRowFactor;
+typedef struct {
+    float* x;             // float32 residual stream [M, N], updated in place
+    int ldx;
+    const float* weight;  // [N] the following norm's weight
+    float alpha;          // x += alpha * result
+    float* sumsq_out;     // [n_parts, 16]
+    int n_parts;          // must equal ic_gemm_nt_residual_parts(N)
+} IcResidualNorm;
 // C[M, N] = alpha * A[M, K] W[N, K]^T, bfloat16 operands, float32 accumulation.  c_mode 1 (M <= 16):
-// W = [gate; up], C[M, N/2] = up * silu(gate).
+// W = [gate; up], C[M, N/2] = up * silu(gate).  c_mode 2 (M <= 16, bfloat16 C, tail != NULL):
+// x += tail->alpha * (alpha A W^T), C = x * tail->weight.  row_factor (nullable, M <= 16): see above.
 int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype);
-int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode, hipStream_t stream);
+int ic_gemm_nt_residual_parts(int N);
+int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode, const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream);
 // The same with the tiling chosen by the caller (tuning and tests); nt == 0 selects the SwiGLU variant.
 int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int nt, int wpb, int unroll, hipStream_t stream);
-// QKV projection of M <= 16 rows with rotary and cache write in the epilogue.
+// QKV projection of M <= 16 rows with rotary and cache write in the epilogue; row_factor nullable.
 int ic_gemm_qkv_rope_supported(int dtype, int dh);
-int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc, const int* positions, const int* slots, const float* cos_t, const float* sin_t, void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size, hipStream_t stream);
+int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc, const int* positions, const int* slots, const float* cos_t, const float* sin_t, void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size, const IcRowFactor* row_factor, hipStream_t stream);
 
 // ---- sampling.hip -----------------------------------------------------------------------------------
 // Greedy choice per row; scratch_val / scratch_idx: 64 * n_rows elements.

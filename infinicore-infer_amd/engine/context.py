@@ -61,6 +61,7 @@ class StepContext:
         self.state_slots = None          # int32 [R]  state slot of each request
         self.want_rows = None            # int32 [W]  token rows whose logits are wanted
         self.n_want = 0
+        self.want_rows_identity = False  # every row's logits are wanted, in order
         self.decode_rows = None          # int32 [n_decode_rows] rows that are a request's single token
         self.n_decode_rows = 0
         self.decode_rows_identity = False

@@ -278,6 +278,7 @@ class Engine:
         ctx.tokens, ctx.positions, ctx.token_req = view("tokens"), view("positions"), view("token_req")
         ctx.state_slots = view("state_slots")
         ctx.want_rows, ctx.n_want = view("want_rows"), len(want_rows)
+        ctx.want_rows_identity = (len(want_rows) == T and all(w == i for i, w in enumerate(want_rows)))
         ctx.decode_rows, ctx.n_decode_rows = view("decode_rows"), len(decode_rows)
         ctx.decode_rows_identity = (len(decode_rows) == T)
         ctx.prefill_tiles = view("tiles").view(-1, 4)
@@ -407,7 +408,7 @@ class _DecodeGraph:
         ctx.T, ctx.R, ctx.page_size, ctx.ws = R, R, engine.page_size, Workspace(engine.device)
         ctx.tokens, ctx.positions, ctx.token_req = view("tokens"), view("positions"), view("token_req")
         ctx.state_slots = view("state_slots")
-        ctx.want_rows, ctx.n_want = view("want_rows"), R
+        ctx.want_rows, ctx.n_want, ctx.want_rows_identity = view("want_rows"), R, True
         ctx.decode_rows, ctx.n_decode_rows, ctx.decode_rows_identity = None, R, True
         ctx.prefill_tiles, ctx.n_prefill_tiles = None, 0
         ctx.req_start = list(range(R + 1))

@@ -25,6 +25,21 @@ _I = _c.c_int
 _F = _c.c_float
 _LL = _c.c_longlong
 
+
+
+class IcRowFactor(_c.Structure):
+    """Row factors rsqrt(sum / width + eps) owed by the rows of an operand (see the C header)."""
+    _fields_ = [("sumsq", _P), ("n_parts", _I), ("width", _I), ("eps", _F)]
+
+
+class IcResidualNorm(_c.Structure):
+    """Residual add and norm weight in a product's epilogue (see the C header)."""
+    _fields_ = [("x", _P), ("ldx", _I), ("weight", _P), ("alpha", _F), ("sumsq_out", _P), ("n_parts", _I)]
+
+
+_RF = _c.POINTER(IcRowFactor)
+_RN = _c.POINTER(IcResidualNorm)
+
 _SIGNATURES = {
     "ic_embed": [_P, _P, _I, _P, _I, _I, _F, _P],
     "ic_rmsnorm": [_P, _P, _P, _P, _I, _I, _I, _F, _F, _P],
@@ -40,10 +55,11 @@ _SIGNATURES = {
     "ic_attn_prefill": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
-    "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _P],
+    "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],
+    "ic_gemm_nt_residual_parts": [_I],
     "ic_gemm_nt_supported": [_I, _I, _I],
     "ic_gemm_qkv_rope_supported": [_I, _I],
-    "ic_gemm_qkv_rope": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _P],
+    "ic_gemm_qkv_rope": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _RF, _P],
     "ic_gemm_nt_cfg": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
 }
 

@@ -249,18 +249,62 @@ def gemm_nt_supported(a_dtype, w_dtype, c_dtype) -> bool:
         return False
 
 
-def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False):
+MAX_SUMSQ_PARTS = 256      # column blocks of sums of squares a product can take as row factors
+
+
+def residual_parts(n: int) -> int:
+    """Column blocks of sums of squares that gemm_nt(..., residual=...) writes for an n wide product."""
+    return (n + 15) // 16
+
+
+def _row_factor(row_factor, M, what):
+    """row_factor = (sumsq float32 [n_parts, 16], width, eps) -> the C struct (or None)."""
+    if row_factor is None:
+        return None
+    from .lib import IcRowFactor
+    sumsq, width, eps = row_factor
+    _dev(sumsq)
+    _need(M <= 16, what + ": row factors need at most 16 rows")
+    _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.dim() == 2 and sumsq.shape[1] == 16
+          and 0 < sumsq.shape[0] <= MAX_SUMSQ_PARTS, what + ": sums of squares must be float32 [<= 256, 16]")
+    _need(width > 0, what + ": width")
+    return IcRowFactor(sumsq.data_ptr(), sumsq.shape[0], int(width), float(eps))
+
+
+def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_factor=None, residual=None):
     """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation).
-    swiglu_output (M <= 16): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate)."""
+    swiglu_output (M <= 16): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate).
+    row_factor = (sumsq [n_parts, 16], width, eps), M <= 16: row m of the product is first multiplied by
+    rsqrt(sumsq[:, m].sum() / width + eps), the factor an RMS norm of a's rows still owes.
+    residual = (x float32 [M, N], weight float32 [N], beta, sumsq_out float32 [residual_parts(N), 16]),
+    M <= 16, bfloat16 out: x += beta * (the product rounded to bfloat16); out = x * weight;
+    sumsq_out[b, m] = sum of x[m]^2 over columns 16 b .. 16 b + 15."""
+    import ctypes
     _dev(a, w, out)
     M, K = a.shape
     N = w.shape[0]
     _need(w.shape[1] == K and tuple(out.shape) == (M, N // 2 if swiglu_output else N), "gemm_nt: shape mismatch")
     _need(not swiglu_output or (M <= 16 and N % 2 == 0), "gemm_nt: fused activation needs M <= 16 and even N")
     _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm_nt: inner strides must be 1")
+    rf = _row_factor(row_factor, M, "gemm_nt")
+    rn = None
+    mode = 1 if swiglu_output else 0
+    if residual is not None:
+        from .lib import IcResidualNorm
+        x, weight, beta, sumsq_out = residual
+        _dev(x, weight, sumsq_out)
+        _need(not swiglu_output and M <= 16 and out.dtype == torch.bfloat16, "gemm_nt: residual epilogue needs M <= 16 and bfloat16 out")
+        _need(x.dtype == torch.float32 and tuple(x.shape) == (M, N) and x.stride(1) == 1, "gemm_nt: residual stream must be float32 [M, N]")
+        _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() == N, "gemm_nt: norm weight must be float32 [N]")
+        _need(sumsq_out.dtype == torch.float32 and sumsq_out.is_contiguous()
+              and tuple(sumsq_out.shape) == (residual_parts(N), 16) and residual_parts(N) <= MAX_SUMSQ_PARTS,
+              "gemm_nt: sumsq_out must be float32 [residual_parts(N) <= 256, 16]")
+        rn = IcResidualNorm(x.data_ptr(), x.stride(0), weight.data_ptr(), float(beta), sumsq_out.data_ptr(), sumsq_out.shape[0])
+        mode = 2
     check(get_lib().ic_gemm_nt(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
                                out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),
-                               out.stride(0), float(alpha), 1 if swiglu_output else 0, _stream()), "gemm_nt")
+                               out.stride(0), float(alpha), mode, ctypes.byref(rf) if rf else None,
+                               ctypes.byref(rn) if rn else None, _stream()), "gemm_nt")
     return out
 
 
@@ -271,15 +315,18 @@ def gemm_qkv_rope_supported(dtype, head_dim: int) -> bool:
         return False
 
 
-def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads, n_kv_heads, head_dim, page_size):
+def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads, n_kv_heads, head_dim, page_size,
+                  row_factor=None):
     """For M <= 16 rows: qkv = a @ w^T with the rotary encoding and the cache write in the epilogue.
     The q heads of qkv[M, >= n_heads * head_dim] hold rotated queries afterwards; rotated keys and
-    the values are in cache slot ``slots[m]``.  Full rotary, bfloat16."""
+    the values are in cache slot ``slots[m]``.  Full rotary, bfloat16.  row_factor: as in gemm_nt."""
+    import ctypes
     _dev(a, w, qkv, positions, slots, cos, sin, kcache, vcache)
     M, K = a.shape
     _i32(positions, "positions")
     _i32(slots, "slots")
     _need(M <= 16 and positions.numel() == M and slots.numel() == M, "gemm_qkv_rope: at most 16 rows, one position and slot each")
+    rf = _row_factor(row_factor, M, "gemm_qkv_rope")
     _need(tuple(w.shape) == ((n_heads + 2 * n_kv_heads) * head_dim, K), "gemm_qkv_rope: weight shape")
     _need(qkv.shape[0] == M and qkv.shape[1] >= n_heads * head_dim and qkv.stride(1) == 1
           and a.stride(1) == 1 and w.stride(1) == 1, "gemm_qkv_rope: layout")
@@ -291,5 +338,5 @@ def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads
     check(get_lib().ic_gemm_qkv_rope(a.data_ptr(), w.data_ptr(), qkv.data_ptr(), M, K, a.stride(0), w.stride(0),
                                      qkv.stride(0), positions.data_ptr(), slots.data_ptr(), cos.data_ptr(),
                                      sin.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), n_heads, n_kv_heads,
-                                     head_dim, page_size, _stream()), "gemm_qkv_rope")
+                                     head_dim, page_size, ctypes.byref(rf) if rf else None, _stream()), "gemm_qkv_rope")
     return qkv

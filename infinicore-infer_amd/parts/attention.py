@@ -14,13 +14,15 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import WeightSpec
-from .base import CacheNeed, Mixer, build_part, register_part
-from .linear import linear
+from .base import CacheNeed, DeferredRows, Mixer, build_part, register_part
+from .linear import linear, linear_tail
 
 
 @register_part("mixer", "attention")
 class Attention(Mixer):
     graph_safe = True
+    accepts_deferred = True
+    fuses_tail = True
 
     def __init__(self, name, runtime, hidden_size: int, num_heads: int, num_kv_heads: int, head_dim: int,
                  softmax_scale: float, position_encoding, window=None, shared_kv: bool = False):
@@ -70,7 +72,7 @@ class Attention(Mixer):
         self.w_o = tensors[n + "o_proj.weight"]
 
     # ---- forward ---------------------------------------------------------------------
-    def forward(self, h, ctx, cache):
+    def forward(self, h, ctx, cache, tail=None):
         rt = self.runtime
         T = h.shape[0]
         nkv = 0 if (self.shared_kv or not cache.writes) else self.nkvh
@@ -81,6 +83,9 @@ class Attention(Mixer):
             self.pos_enc.rotate_and_store(qkv, ctx, cache, self.nh, nkv, self.dh)
         out = ctx.ws.buffer("attn_out", (T, self.nh * self.dh), rt.dtype)
         self._attend(qkv, out, ctx, cache)
+        fused = linear_tail(out, self.w_o, tail, ctx.ws, "mixer_tail", rt.gemm_impl)
+        if fused is not None:
+            return fused
         y = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
         linear(out, self.w_o, y, rt.gemm_impl)
         return y

@@ -42,6 +42,47 @@ class CacheNeed:
     state_dtype: torch.dtype = torch.float32
 
 
+@dataclass
+class DeferredRows:
+    """Rows whose norm is half done.  ``values[r]`` is x[r] * w (the norm's weight is applied, its
+    row factor is not); ``sumsq[b, r]`` are sums of x[r]^2 over column blocks b.  The true row is
+    values[r] * rsqrt(sumsq[:, r].sum() / width + eps).  The row factor commutes with a projection,
+    so a part that takes such rows (``accepts_deferred``) applies it to its first product's result."""
+    values: torch.Tensor
+    sumsq: torch.Tensor                # float32 [n_parts, 16]
+    width: int
+    eps: float
+
+    @property
+    def shape(self):
+        return self.values.shape
+
+    @property
+    def dtype(self):
+        return self.values.dtype
+
+    def row_factor(self):
+        return (self.sumsq, self.width, self.eps)
+
+    def materialize(self):
+        """The normed rows as a plain tensor (slow path for parts of a product that cannot take factors)."""
+        T = self.values.shape[0]
+        f = torch.rsqrt(self.sumsq.sum(0)[:T, None] / self.width + self.eps)
+        return (self.values.to(torch.float32) * f).to(self.values.dtype)
+
+
+@dataclass
+class ResidualTail:
+    """What a block asks of a part's LAST projection (a part with ``fuses_tail``): add the part's
+    output y to the float32 residual stream, x += alpha * y, and hand back the input of the norm
+    that follows (weight, eps) as ``DeferredRows``.  A part that cannot do it for this step returns
+    its plain output and the block does the add and the norm itself."""
+    x: torch.Tensor
+    alpha: float
+    weight: torch.Tensor
+    eps: float
+
+
 def register_part(category: str, kind: str) -> Callable:
     if category not in _REGISTRY:
         raise KeyError("unknown part category %r (have %s)" % (category, ", ".join(CATEGORIES)))
@@ -108,6 +149,11 @@ class Norm(Part):
         ops.residual_add(x, y, alpha)
         return self.forward(x, out)
 
+    def deferred(self):
+        """(weight, eps) when the norm is y = x * rsqrt(mean(x^2) + eps) * weight, so that it can be
+        split over the products before and after it (``DeferredRows``); None otherwise."""
+        return None
+
 
 class PositionEncoding(Part):
     category = "position_encoding"
@@ -125,6 +171,8 @@ class PositionEncoding(Part):
 
 class Mixer(Part):
     category = "mixer"
+    accepts_deferred = False     # forward() takes DeferredRows as h
+    fuses_tail = False           # forward() takes tail=ResidualTail and may return DeferredRows
 
     def cache_need(self) -> CacheNeed:
         return CacheNeed()
@@ -136,6 +184,8 @@ class Mixer(Part):
 
 class FeedForward(Part):
     category = "feed_forward"
+    accepts_deferred = False
+    fuses_tail = False
 
     def forward(self, h, ctx):
         raise NotImplementedError
@@ -156,6 +206,15 @@ class Block(Part):
 
     def sub_parts(self):
         return (self.mixer, self.mixer_norm, self.feed_forward, self.feed_forward_norm)
+
+    # A block with ``fuses_successor`` is called as forward(x, pending, ctx, cache, successor=norm):
+    # ``successor`` is the norm that whoever runs next applies first (None: unknown or not splittable),
+    # and the block may return DeferredRows for it instead of a pending add.  ``entry_norm()`` names
+    # the norm a block applies to the incoming stream when it takes DeferredRows as ``pending``.
+    fuses_successor = False
+
+    def entry_norm(self):
+        return None
 
     def forward(self, x, pending, ctx, cache):
         raise NotImplementedError

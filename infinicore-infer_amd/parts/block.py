@@ -5,27 +5,52 @@ is a float32 factor of the residual add).  The layer body is
 src/models/jiuge/jiuge.cpp:195-258.
 
 The residual stream is float32.  Each add is fused with the norm that follows
-it: the block leaves its last add pending for whoever normalises next.
+it: the block leaves its last add pending for whoever normalises next.  For
+few rows the add and the norm go further, into the products on either side
+(``ResidualTail`` / ``DeferredRows``): then a layer is six kernels, not eight.
 """
-from .base import Block, register_part
+from .base import Block, DeferredRows, ResidualTail, register_part
 
 
 @register_part("block", "prenorm_residual")
 class PreNormResidualBlock(Block):
     graph_safe = True
+    fuses_successor = True
 
     def __init__(self, name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm,
                  residual_scale: float = 1.0):
         super().__init__(name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm)
         self.residual_scale = float(residual_scale)
 
-    def forward(self, x, pending, ctx, cache):
-        h = ctx.ws.buffer("normed", tuple(x.shape), self.runtime.dtype)
-        if pending is None:
-            self.mixer_norm.forward(x, h)
+    def entry_norm(self):
+        """The norm applied to the incoming stream, if the mixer can take its rows half done."""
+        return self.mixer_norm if getattr(self.mixer, "accepts_deferred", False) else None
+
+    def _tail(self, producer, consumer_ok, norm, x):
+        """The request to fuse (add, norm) into the producer's last projection, when all three agree."""
+        if not (getattr(producer, "fuses_tail", False) and consumer_ok and norm is not None):
+            return None
+        d = norm.deferred()
+        return None if d is None else ResidualTail(x, self.residual_scale, d[0], d[1])
+
+    def forward(self, x, pending, ctx, cache, successor=None):
+        if isinstance(pending, DeferredRows):
+            h = pending                               # the add is done; the mixer applies the row factors
         else:
-            self.mixer_norm.forward_add(x, pending[0], pending[1], h)
-        y = self.mixer.forward(h, ctx, cache)
-        self.feed_forward_norm.forward_add(x, y, self.residual_scale, h)
-        y = self.feed_forward.forward(h, ctx)
+            h = ctx.ws.buffer("normed", tuple(x.shape), self.runtime.dtype)
+            if pending is None:
+                self.mixer_norm.forward(x, h)
+            else:
+                self.mixer_norm.forward_add(x, pending[0], pending[1], h)
+        tail = self._tail(self.mixer, getattr(self.feed_forward, "accepts_deferred", False), self.feed_forward_norm, x)
+        y = self.mixer.forward(h, ctx, cache, tail=tail) if tail is not None else self.mixer.forward(h, ctx, cache)
+        if isinstance(y, DeferredRows):
+            h = y
+        else:
+            h = ctx.ws.buffer("normed", tuple(x.shape), self.runtime.dtype)
+            self.feed_forward_norm.forward_add(x, y, self.residual_scale, h)
+        tail = self._tail(self.feed_forward, True, successor, x)
+        y = self.feed_forward.forward(h, ctx, tail=tail) if tail is not None else self.feed_forward.forward(h, ctx)
+        if isinstance(y, DeferredRows):
+            return y
         return (y, self.residual_scale)

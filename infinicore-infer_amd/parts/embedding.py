@@ -43,6 +43,7 @@ class Embedding(Part):
 @register_part("head", "lm_head")
 class LMHead(Part):
     graph_safe = True
+    accepts_deferred = True
 
     category = "head"
 
@@ -62,6 +63,11 @@ class LMHead(Part):
 
     def forward(self, x, rows, final_norm, ctx):
         """Float32 logits [len(rows), vocab] of the residual rows ``rows``."""
+        from .base import DeferredRows
+        if isinstance(x, DeferredRows):
+            # every row in order, the final norm half done: its row factors go into the product
+            logits = ctx.ws.buffer("logits", (x.shape[0], self.vocab_size), torch.float32)
+            return linear(x, self.weight, logits, self.runtime.gemm_impl, alpha=self.logit_scale)
         n = rows.numel()
         h = ctx.ws.buffer("head_in", (n, self.hidden_size), self.runtime.dtype)
         final_norm.forward(x, h, rows=rows, out_scale=self.logit_scale)

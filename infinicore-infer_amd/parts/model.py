@@ -13,7 +13,7 @@ import torch
 from ..config.spec import ModelSpec
 from ..kernels import ops
 from ..weights.loader import WeightSpec, load_weights
-from .base import CacheNeed, Runtime, build_part
+from .base import CacheNeed, DeferredRows, Runtime, build_part
 
 
 class DecoderModel:
@@ -112,10 +112,26 @@ class DecoderModel:
         x = ctx.ws.buffer("residual", (T, self.spec.hidden_size), torch.float32)
         self.embedding.forward(ctx.tokens, x)
         pending = None
-        for e in self.schedule:
-            pending = self.layers[e.layer].forward(x, pending, ctx, ctx.cache_view(e))
+        last = len(self.schedule) - 1
+        for i, e in enumerate(self.schedule):
+            block = self.layers[e.layer]
+            if not block.fuses_successor:
+                if isinstance(pending, DeferredRows):
+                    raise RuntimeError("block %s was handed half-normed rows it did not ask for" % block.name)
+                pending = block.forward(x, pending, ctx, ctx.cache_view(e))
+                continue
+            # the norm that runs next, if whoever applies it can take its rows half done
+            if i < last:
+                successor = self.layers[self.schedule[i + 1].layer].entry_norm()
+            elif ctx.want_rows_identity and getattr(self.head, "accepts_deferred", False):
+                successor = self.final_norm
+            else:
+                successor = None
+            pending = block.forward(x, pending, ctx, ctx.cache_view(e), successor=successor)
         if ctx.n_want == 0:
             return None
+        if isinstance(pending, DeferredRows):
+            return self.head.forward(pending, ctx.want_rows, self.final_norm, ctx)
         if pending is not None:
             ops.residual_add(x, pending[0], pending[1])
         return self.head.forward(x, ctx.want_rows, self.final_norm, ctx)

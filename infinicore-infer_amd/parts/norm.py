@@ -28,3 +28,6 @@ class RMSNorm(Norm):
 
     def forward_add(self, x, y, alpha, out):
         return ops.add_rmsnorm(x, y, alpha, self.weight, out, self.eps)
+
+    def deferred(self):
+        return (self.weight, self.eps)

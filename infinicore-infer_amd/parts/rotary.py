@@ -71,8 +71,12 @@ class Rotary(PositionEncoding):
 
     def project_rotate_store(self, h, w_qkv, qkv, ctx, cache, n_heads, n_kv_heads, head_dim) -> bool:
         """Few rows in bfloat16 with full rotary: the projection kernel rotates and writes the cache."""
+        from .base import DeferredRows
         from .linear import FEW_ROWS
         rt = self.runtime
+        row_factor = None
+        if isinstance(h, DeferredRows):
+            h, row_factor = h.values, h.row_factor()
         if (h.shape[0] > FEW_ROWS or rt.gemm_impl != "auto" or n_kv_heads == 0 or self.rot_dim != head_dim
                 or h.dtype != torch.bfloat16 or w_qkv.dtype != torch.bfloat16
                 or not ops.gemm_qkv_rope_supported(h.dtype, head_dim)):
@@ -80,7 +84,7 @@ class Rotary(PositionEncoding):
         if ctx.max_position >= self.max_positions:
             raise ValueError("position %d is beyond the rotary tables (%d)" % (ctx.max_position, self.max_positions))
         ops.gemm_qkv_rope(h, w_qkv, qkv, ctx.positions, cache.slots, self.cos, self.sin, cache.k, cache.v,
-                          n_heads, n_kv_heads, head_dim, ctx.page_size)
+                          n_heads, n_kv_heads, head_dim, ctx.page_size, row_factor=row_factor)
         return True
 
 

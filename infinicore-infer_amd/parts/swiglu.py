@@ -9,13 +9,15 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import WeightSpec
-from .base import FeedForward, register_part
-from .linear import FEW_ROWS, linear
+from .base import DeferredRows, FeedForward, register_part
+from .linear import linear, linear_tail, own_kernel_applies
 
 
 @register_part("feed_forward", "swiglu")
 class SwiGLU(FeedForward):
     graph_safe = True
+    accepts_deferred = True
+    fuses_tail = True
 
     def __init__(self, name, runtime, hidden_size: int, intermediate_size: int):
         super().__init__(name, runtime)
@@ -40,18 +42,23 @@ class SwiGLU(FeedForward):
         self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = tensors[n + "down_proj.weight"]
 
-    def forward(self, h, ctx):
+    def forward(self, h, ctx, tail=None):
         rt = self.runtime
         T = h.shape[0]
         act = ctx.ws.buffer("ffn_act", (T, self.intermediate_size), rt.dtype)
-        if (T <= FEW_ROWS and rt.gemm_impl == "auto" and self.w_gate_up.dtype == h.dtype
-                and ops.gemm_nt_supported(h.dtype, self.w_gate_up.dtype, act.dtype)):
+        if own_kernel_applies(T, h.dtype, self.w_gate_up.dtype, act.dtype, rt.gemm_impl):
             # few rows: the activation is the epilogue of the gate/up projection
-            ops.gemm_nt(h, self.w_gate_up, act, swiglu_output=True)
+            if isinstance(h, DeferredRows):
+                ops.gemm_nt(h.values, self.w_gate_up, act, swiglu_output=True, row_factor=h.row_factor())
+            else:
+                ops.gemm_nt(h, self.w_gate_up, act, swiglu_output=True)
         else:
             gate_up = ctx.ws.buffer("gate_up", (T, 2 * self.intermediate_size), rt.dtype)
             linear(h, self.w_gate_up, gate_up, rt.gemm_impl)
             ops.swiglu(gate_up, act)
+        fused = linear_tail(act, self.w_down, tail, ctx.ws, "ffn_tail", rt.gemm_impl)
+        if fused is not None:
+            return fused
         y = ctx.ws.buffer("ffn_out", (T, self.hidden_size), rt.dtype)
         linear(act, self.w_down, y, rt.gemm_impl)
         return y

@@ -433,3 +433,78 @@ def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page):
     _close(kc, kc2, torch.bfloat16)
     _close(vc, vc2, torch.bfloat16)
     assert float(kc2.abs().max()) > 0 and float(vc2.abs().max()) > 0
+
+
+@pytest.mark.parametrize("M,N,K,N2", [(1, 200, 344, 331), (8, 2304, 2304, 6912), (16, 96, 509, 64), (5, 4096, 130, 50),
+                                      (3, 1536, 3840, 1000)])
+def test_norm_split_over_two_products(M, N, K, N2):
+    """Residual add + RMS norm between two products, split over them: the first product's
+    epilogue adds to the stream and stores x * w with sums of squares; the second applies the
+    row factors to its result.  Equals product, add, norm, product done one after the other."""
+    g = torch.Generator().manual_seed(41)
+    ops = _ops()
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w1 = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16)
+    w2 = (torch.randn(N2, N, generator=g) * 0.1).to(torch.bfloat16)
+    x = torch.randn(M, N, generator=g) * 3.0
+    gw = torch.rand(N, generator=g) + 0.5
+    beta, eps, alpha2 = 0.37, 1e-5, 0.7
+    xd = x.to(DEV)
+    y = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    sumsq = torch.full((ops.residual_parts(N), 16), float("nan"), device=DEV)
+    ops.gemm_nt(a.to(DEV), w1.to(DEV), y, residual=(xd, gw.to(DEV), beta, sumsq))
+    # the stream after the add: the product is rounded to bfloat16 before it is added, so the stream
+    # may differ from the exact sum by that rounding (relative to the product), no more
+    delta = P.plain_linear(a, w1)
+    _close(xd, x.double() + beta * delta, torch.bfloat16, scale=beta * float(delta.abs().max()))
+    assert float((xd.cpu() - x).abs().max()) > 0
+    # the half-done rows and the sums follow from the stream as it now is
+    x_new = xd.double().cpu()
+    _close(y, x_new * gw.double(), torch.bfloat16)
+    ss = sumsq.double().cpu()
+    assert torch.isfinite(ss).all()
+    assert float(ss[:, M:].abs().max()) == 0.0 if M < 16 else True      # rows that do not exist add nothing
+    _close(ss.sum(0)[:M], (x_new * x_new).sum(1), torch.float32, factor=10)
+    # second product with the row factors, float32 and bfloat16 results
+    for cdtype in DT:
+        out = torch.empty(M, N2, dtype=cdtype, device=DEV)
+        ops.gemm_nt(y, w2.to(DEV), out, alpha=alpha2, row_factor=(sumsq, N, eps))
+        rs = torch.rsqrt((x_new * x_new).mean(1, keepdim=True) + eps)
+        want = alpha2 * rs * P.plain_linear(y.cpu(), w2)
+        _close(out, want, cdtype, factor=1 if cdtype == torch.bfloat16 else 100)
+        # and it is the norm: compare with norm-then-product in float64 (bf16 rounding of the rows apart)
+        full = alpha2 * P.plain_linear(P.plain_rmsnorm(x_new, gw, eps), w2)
+        _close(out, full, torch.bfloat16, factor=2)
+    # the activation and the rotary epilogues take the factors too
+    if N2 % 2 == 0:
+        act = torch.empty(M, N2 // 2, dtype=torch.bfloat16, device=DEV)
+        ops.gemm_nt(y, w2.to(DEV), act, swiglu_output=True, row_factor=(sumsq, N, eps))
+        gu = P.round_bf16(rs * P.plain_linear(y.cpu(), w2))
+        _close(act, P.plain_swiglu(gu[:, :N2 // 2], gu[:, N2 // 2:]), torch.bfloat16, factor=2)
+
+
+def test_gemm_qkv_rope_with_row_factors():
+    g = torch.Generator().manual_seed(43)
+    ops = _ops()
+    M, nh, nkvh, dh, K, page = 7, 6, 2, 64, 200, 16
+    H = (nh + 2 * nkvh) * dh
+    yv = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(H, K, generator=g) * 0.1).to(torch.bfloat16)
+    sumsq = (torch.rand(ops.residual_parts(K), 16, generator=g) * 4.0).to(DEV)
+    eps = 1e-6
+    rs = torch.rsqrt(sumsq.double().cpu().sum(0)[:M, None] / K + eps)
+    pos = torch.randint(0, 300, (M,), generator=g, dtype=torch.int32)
+    slots = torch.randperm(5 * page, generator=g)[:M].to(torch.int32)
+    sin, cos = P.plain_rope_tables(dh, 10000.0, 300)
+    sin, cos = sin.float().to(DEV), cos.float().to(DEV)
+    kc = torch.zeros(5, nkvh, page, dh, dtype=torch.bfloat16, device=DEV)
+    vc = torch.zeros_like(kc)
+    qkv = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
+    ops.gemm_qkv_rope(yv.to(DEV), w.to(DEV), qkv, pos.to(DEV), slots.to(DEV), cos, sin, kc, vc, nh, nkvh, dh, page,
+                      row_factor=(sumsq, K, eps))
+    ref = P.round_bf16(rs * P.plain_linear(yv, w)).to(torch.bfloat16).to(DEV)
+    kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
+    ops.rope_kv_write(ref, pos.to(DEV), cos, sin, kc2, vc2, slots.to(DEV), nh, nkvh, dh, dh, page)
+    _close(qkv[:, :nh * dh], ref[:, :nh * dh], torch.bfloat16)
+    _close(kc, kc2, torch.bfloat16)
+    _close(vc, vc2, torch.bfloat16)
