@@ -50,7 +50,7 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* acc, int 
     m = mn;
 }
 
-template <typename T, int DH, int GQ>
+template <typename T, int DH, int GQ, bool STAGED>
 __global__ void __launch_bounds__(kDecThreads)
 attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
                          const T* __restrict__ kcache, const T* __restrict__ vcache,
@@ -89,18 +89,20 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
     const T* kbase = kcache + (size_t)kvh * head_stride + sub * VEC;
     const T* vbase = vcache + (size_t)kvh * head_stride + sub * VEC;
 
-    // page ids of this block's keys, staged once: the loop then needs one memory hop per key
+    // page ids of this block's keys, staged once: the loop then needs one memory hop per key.
+    // STAGED is a compile-time choice (the host knows the block table's width): a run-time choice
+    // between the two arrays would make every lookup a flat load, whose wait also waits for the
+    // key and value loads in flight.
     const int page_lo = lo / page_size;
     const int n_pages = (hi > lo) ? (hi - 1) / page_size - page_lo + 1 : 0;
-    const bool staged = n_pages <= kDecMaxPages;
-    if (staged)
+    if (STAGED)
         for (int i = threadIdx.x; i < n_pages; i += kDecThreads) pages[i] = bt[page_lo + i];
     __syncthreads();
 
     // element offset of a key's row piece in a plane
     auto row_of = [&](int key) -> size_t {
         const int lp = key / page_size;
-        const int pg = staged ? pages[lp - page_lo] : bt[lp];
+        const int pg = STAGED ? pages[lp - page_lo] : bt[lp];
         return (size_t)pg * page_stride + (size_t)(key - lp * page_size) * DH;
     };
 
@@ -277,7 +279,7 @@ union GqFrag {
     gq_bf16x8 v;
 };
 
-template <int DH>
+template <int DH, bool STAGED>
 __global__ void __launch_bounds__(kDecThreads)
 attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
                        const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
@@ -317,13 +319,12 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
 
     const int page_lo = lo / page_size;
     const int n_pages = (hi > lo) ? (hi - 1) / page_size - page_lo + 1 : 0;
-    const bool staged = n_pages <= kDecMaxPages;
-    if (staged)
+    if (STAGED)
         for (int i = threadIdx.x; i < n_pages; i += kDecThreads) pages[i] = bt[page_lo + i];
     __syncthreads();
     auto row_of = [&](int key) -> size_t {
         const int lp = key / page_size;
-        const int pg = staged ? pages[lp - page_lo] : bt[lp];
+        const int pg = STAGED ? pages[lp - page_lo] : bt[lp];
         return (size_t)pg * page_stride + (size_t)(key - lp * page_size) * DH;
     };
 
@@ -479,18 +480,22 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
                          int n_tok, int nh, int nkvh, int page_size, float scale, int window, int nsplit,
                          hipStream_t stream) {
     dim3 grid(nsplit, nkvh, n_tok), block(kDecThreads);
-    if (nh != nkvh && sizeof(T) == 2)
-        hipLaunchKernelGGL((attn_decode_gqa_kernel<DH>), grid, block, 0, stream, (const uint16_t*)q, q_stride,
-                           (const uint16_t*)kcache, (const uint16_t*)vcache, block_tables, bt_stride, tok_list,
-                           token_req, positions, part_acc, part_ml, nh, nkvh, page_size, scale, window, nsplit);
-    else if (nh == nkvh)
-        hipLaunchKernelGGL((attn_decode_split_kernel<T, DH, 1>), grid, block, 0, stream, (const T*)q, q_stride,
-                           (const T*)kcache, (const T*)vcache, block_tables, bt_stride, tok_list, token_req,
-                           positions, part_acc, part_ml, nh, nkvh, page_size, scale, window, nsplit);
-    else
-        hipLaunchKernelGGL((attn_decode_split_kernel<T, DH, 4>), grid, block, 0, stream, (const T*)q, q_stride,
-                           (const T*)kcache, (const T*)vcache, block_tables, bt_stride, tok_list, token_req,
-                           positions, part_acc, part_ml, nh, nkvh, page_size, scale, window, nsplit);
+    const bool staged = bt_stride <= kDecMaxPages;      // a block never needs more page ids than a request has
+#define IC_DEC_LAUNCH(KERNEL, TQ)                                                                           \
+    hipLaunchKernelGGL(KERNEL, grid, block, 0, stream, (const TQ*)q, q_stride, (const TQ*)kcache,           \
+                       (const TQ*)vcache, block_tables, bt_stride, tok_list, token_req, positions, part_acc, \
+                       part_ml, nh, nkvh, page_size, scale, window, nsplit)
+    if (nh != nkvh && sizeof(T) == 2) {
+        if (staged) IC_DEC_LAUNCH((attn_decode_gqa_kernel<DH, true>), uint16_t);
+        else IC_DEC_LAUNCH((attn_decode_gqa_kernel<DH, false>), uint16_t);
+    } else if (nh == nkvh) {
+        if (staged) IC_DEC_LAUNCH((attn_decode_split_kernel<T, DH, 1, true>), T);
+        else IC_DEC_LAUNCH((attn_decode_split_kernel<T, DH, 1, false>), T);
+    } else {
+        if (staged) IC_DEC_LAUNCH((attn_decode_split_kernel<T, DH, 4, true>), T);
+        else IC_DEC_LAUNCH((attn_decode_split_kernel<T, DH, 4, false>), T);
+    }
+#undef IC_DEC_LAUNCH
     int st = ic_launch_status();
     if (st) return st;
     hipLaunchKernelGGL(attn_decode_reduce_kernel<T>, dim3(n_tok * nh), dim3(64), 0, stream, part_acc, part_ml,

@@ -1,10 +1,14 @@
 // Attention of prompt portions over the paged cache on the matrix cores
 // (bfloat16 operands, float32 accumulation and softmax).
 //
-// Grid (8 * ceil(heads / 8) * query tiles), 256 threads, dealt to the XCDs head by head.  A tile is up to 128 consecutive
-// tokens of one request; wave w owns rows 32w..32w+31.  Keys and values come
-// in tiles of 64 through LDS (values transposed on the way in); the next tile
-// is already on its way from memory while the current one is used.  Scores
+// Grid (8 * ceil(heads / 8) * query tiles), 256 * GROUPS threads, dealt to the XCDs head by head.  A tile is up to 128
+// consecutive tokens of one request; wave w of a group owns rows 32w..32w+31.  With GROUPS == 2
+// the two groups take the even and the odd key tiles of 64 and are merged through LDS at the
+// end: the longest query tile of a prompt, which sets the kernel's time when there are few
+// blocks, then walks half as many key tiles.  With many blocks GROUPS == 1 keeps more of them
+// resident and is faster.  Keys and values come through LDS, 64 * GROUPS keys a step (values
+// transposed on the way in); the next step is already on its way from memory while the
+// current one is used.  Scores
 // are computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: every
 // lane then holds 32 keys of ONE query, so the running softmax needs a single
 // cross-lane step, and the probabilities are already laid out as the B operand
@@ -23,7 +27,7 @@ typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v8f __attribute__((ext_vector_type(8)));
 
-constexpr int kPfThreads = 256;
+constexpr int kPfWaveThreads = 256;   // four waves own the 128 rows of a query tile
 constexpr int kPfRows = 128;      // query rows per block
 constexpr int kPfKeys = 64;       // keys per tile
 constexpr int kPfPad = 8;         // elements of padding per LDS row
@@ -35,8 +39,8 @@ union Frag8 {
     bf16x8 v;
 };
 
-template <int DH>
-__global__ void __launch_bounds__(kPfThreads, (DH <= 64 ? 3 : 1))
+template <int DH, bool STAGED, int GROUPS>
+__global__ void __launch_bounds__(256 * GROUPS, (GROUPS == 1 && DH <= 64) ? 3 : 2)
 attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                          const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                          const int* __restrict__ block_tables, int bt_stride, const int4* __restrict__ tiles,
@@ -45,9 +49,15 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     constexpr int ND = DH / 32;           // 32-row tiles of O^T
     constexpr int KS = DH + kPfPad;       // row stride of Ks (elements)
     constexpr int VS = kPfKeys + kPfPad;  // row stride of Vt
-    constexpr int NL = kPfKeys * (DH / 8) / kPfThreads;   // 16-byte loads per thread per plane and tile
-    __shared__ __attribute__((aligned(16))) uint16_t Ks[kPfKeys * KS];
-    __shared__ __attribute__((aligned(16))) uint16_t Vt[DH * VS];
+    constexpr int kPfThreads = kPfWaveThreads * GROUPS;
+    constexpr int STEP = kPfKeys * GROUPS;                 // keys staged per step
+    constexpr int NL = STEP * (DH / 8) / kPfThreads;       // 16-byte loads per thread per plane and step
+    constexpr int KT = kPfKeys * KS, VT = DH * VS;         // elements of one group's K and V^T tile
+    constexpr int MERGE_F = 2 + ND * 16;                   // floats a lane hands over at the end
+    static_assert(GROUPS == 1 || sizeof(uint16_t) * GROUPS * (KT + VT) >= sizeof(float) * 256 * MERGE_F, "merge buffer fits in the tiles");
+    __shared__ __attribute__((aligned(16))) uint16_t tilebuf[GROUPS * (KT + VT)];
+    uint16_t* const Ks_all = tilebuf;                      // [group][key][KS]
+    uint16_t* const Vt_all = tilebuf + GROUPS * KT;     // [group][dim][VS]
 
     __shared__ int pages[kPfMaxPages];
 
@@ -60,7 +70,8 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     const int req = tile.x, row0 = tile.y, n_rows = tile.z, pos0 = tile.w;
     const int kvh = h / (nh / nkvh);
     const int* bt = block_tables + (size_t)req * bt_stride;
-    const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
+    const int tid = threadIdx.x, lane = tid & 63;
+    const int grp = tid >> 8, wave = (tid >> 6) & 3;        // key-tile group, and the 32 rows this wave owns
     const int lq = lane & 31, half = lane >> 5;
     const int page_size = 1 << page_shift, page_mask = page_size - 1;     // pages are a power of two here
 
@@ -76,11 +87,13 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
 
     // page ids of the keys this block reads, staged once (one memory hop less per tile)
     const int page_lo = first_key >> page_shift, page_hi = last_key >> page_shift;
-    const bool staged = page_hi - page_lo < kPfMaxPages;
-    if (staged)
+    // STAGED is chosen by the host from the block table's width: a run-time choice between the
+    // two arrays would turn every lookup into a flat load, and waiting for a flat load also
+    // waits for the key and value loads in flight.
+    if (STAGED)
         for (int i = tid; i <= page_hi - page_lo; i += kPfThreads) pages[i] = bt[page_lo + i];
     __syncthreads();
-    auto page_of = [&](int ka) -> int { return staged ? pages[(ka >> page_shift) - page_lo] : bt[ka >> page_shift]; };
+    auto page_of = [&](int ka) -> int { return STAGED ? pages[(ka >> page_shift) - page_lo] : bt[ka >> page_shift]; };
 
     // Q^T fragments: Q[query lq][16c + 8 half .. +7]
     Frag8 qf[NC];
@@ -122,7 +135,7 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                 }
             }
             {
-                const int oct = idx / kPfKeys, key = idx - oct * kPfKeys;
+                const int oct = idx / STEP, key = idx - oct * STEP;
                 const int ka = kt + key;
                 vreg[i] = make_uint4(0, 0, 0, 0);
                 if (ka <= last_key && ka >= first_key) {
@@ -138,12 +151,12 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             const int idx = tid + i * kPfThreads;
             {
                 const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
-                *reinterpret_cast<uint4*>(&Ks[key * KS + oct * 8]) = kreg[i];
+                *reinterpret_cast<uint4*>(&Ks_all[(key / kPfKeys) * KT + (key % kPfKeys) * KS + oct * 8]) = kreg[i];
             }
             {
-                const int oct = idx / kPfKeys, key = idx - oct * kPfKeys;
+                const int oct = idx / STEP, key = idx - oct * STEP;
                 const uint4 v = vreg[i];
-                uint16_t* vp = &Vt[(oct * 8) * VS + key];
+                uint16_t* vp = &Vt_all[(key / kPfKeys) * VT + (oct * 8) * VS + (key % kPfKeys)];
                 vp[0 * VS] = (uint16_t)(v.x & 0xffff); vp[1 * VS] = (uint16_t)(v.x >> 16);
                 vp[2 * VS] = (uint16_t)(v.y & 0xffff); vp[3 * VS] = (uint16_t)(v.y >> 16);
                 vp[4 * VS] = (uint16_t)(v.z & 0xffff); vp[5 * VS] = (uint16_t)(v.z >> 16);
@@ -152,13 +165,16 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         }
     };
 
+    const uint16_t* const Ks = Ks_all + grp * KT;
+    const uint16_t* const Vt = Vt_all + grp * VT;
     const int kt0 = (first_key / kPfKeys) * kPfKeys;
     fetch(kt0);
-    for (int kt = kt0; kt <= last_key; kt += kPfKeys) {
-        __syncthreads();                                     // the previous tile's readers are done
+    for (int kb = kt0; kb <= last_key; kb += STEP) {
+        __syncthreads();                                     // the previous step's readers are done
         stash();
         __syncthreads();
-        if (kt + kPfKeys <= last_key) fetch(kt + kPfKeys);   // in flight while this tile is used
+        if (kb + STEP <= last_key) fetch(kb + STEP);         // in flight while this step is used
+        const int kt = kb + kPfKeys * grp;                   // this group's key tile
         if (!wave_ok || kt > wave_last) continue;            // nothing this wave may see
         if (window > 0 && kt + kPfKeys - 1 < wave_first - window + 1) continue;
 
@@ -236,6 +252,31 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         }
     }
 
+    // ---- the odd-tile group hands its state to the even-tile group (same lane, same rows) ----------
+    if (GROUPS == 2) {
+    __syncthreads();                                         // every wave is done with the tiles
+    float* const mbuf = reinterpret_cast<float*>(tilebuf) + (size_t)(wave * 64 + lane) * MERGE_F;
+    if (grp == 1) {
+        mbuf[0] = m; mbuf[1] = l;
+#pragma unroll
+        for (int i = 0; i < ND; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) mbuf[2 + 16 * i + r] = oacc[i][r];
+    }
+    __syncthreads();
+    if (grp == 1) return;
+    {
+        const float m1 = mbuf[0], l1 = mbuf[1];
+        const float m_new = fmaxf(m, m1);
+        const float mc = ((m_new == -INFINITY) ? 0.f : m_new) * scale_log2e;
+        const float c0 = __builtin_amdgcn_exp2f(m * scale_log2e - mc), c1 = __builtin_amdgcn_exp2f(m1 * scale_log2e - mc);
+        l = l * c0 + l1 * c1;
+#pragma unroll
+        for (int i = 0; i < ND; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) oacc[i][r] = oacc[i][r] * c0 + mbuf[2 + 16 * i + r] * c1;
+    }
+    }
     if (!row_ok) return;
     const float inv = 1.0f / l;
     uint16_t* op = out + (size_t)(row0 + my_row) * out_stride + (size_t)h * DH;
@@ -270,15 +311,27 @@ IC_EXPORT int ic_attn_prefill(const void* q, int q_stride, void* out, int out_st
     if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7) ||
         ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15) || ((uintptr_t)tiles & 15)) return IC_ERR_ARG;
     const float sl2 = scale * 1.4426950408889634f;
-    dim3 grid(8 * ((nh + 7) / 8) * n_tiles), block(kPfThreads);
-    if (dh == 64)
-        hipLaunchKernelGGL(attn_prefill_mfma_kernel<64>, grid, block, 0, stream, (const uint16_t*)q, q_stride,
-                           (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,
-                           block_tables, bt_stride, (const int4*)tiles, n_tiles, nh, nkvh, page_shift, sl2, window);
-    else if (dh == 128)
-        hipLaunchKernelGGL(attn_prefill_mfma_kernel<128>, grid, block, 0, stream, (const uint16_t*)q, q_stride,
-                           (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,
-                           block_tables, bt_stride, (const int4*)tiles, n_tiles, nh, nkvh, page_shift, sl2, window);
+    const bool staged = bt_stride <= kPfMaxPages;       // a block never needs more page ids than a request has
+    // Few blocks (up to 6 per compute unit, measured): the longest tile's walk over the keys sets the
+    // time, so two wave groups share it.  Many blocks: one group, more blocks resident.
+    static int cus = 0;                                 // compute units of the device, asked once
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+        else cus = 256;
+    }
+    const bool two_groups = (long long)nh * n_tiles < 6LL * cus;
+    dim3 grid(8 * ((nh + 7) / 8) * n_tiles);
+#define IC_PF_LAUNCH(DD, ST, GG)                                                                                   \
+    hipLaunchKernelGGL((attn_prefill_mfma_kernel<DD, ST, GG>), grid, dim3(256 * GG), 0, stream, (const uint16_t*)q, \
+                       q_stride, (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
+                       block_tables, bt_stride, (const int4*)tiles, n_tiles, nh, nkvh, page_shift, sl2, window)
+#define IC_PF_GROUPS(DD, ST) do { if (two_groups) IC_PF_LAUNCH(DD, ST, 2); else IC_PF_LAUNCH(DD, ST, 1); } while (0)
+    if (dh == 64) { if (staged) IC_PF_GROUPS(64, true); else IC_PF_GROUPS(64, false); }
+    else if (dh == 128) { if (staged) IC_PF_GROUPS(128, true); else IC_PF_GROUPS(128, false); }
+#undef IC_PF_GROUPS
+#undef IC_PF_LAUNCH
     else
         return IC_ERR_UNSUPPORTED;
     return ic_launch_status();

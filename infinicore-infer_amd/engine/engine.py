@@ -194,7 +194,8 @@ class Engine:
             logits = self._graph_step(entries, starts)
         else:
             ctx = self._build_context(entries, starts)
-            logits = self.model.forward(ctx)
+            with ops.stream_scope():
+                logits = self.model.forward(ctx)
         for e in entries:
             self.cache.trim(e.req_id)
         self.steps_run += 1
@@ -454,13 +455,15 @@ class _DecodeGraph:
     def capture(self, engine):
         """Run the step once eagerly (every buffer then exists and the result is
         already right), then record the same launches."""
-        engine.model.forward(self.ctx)
+        with ops.stream_scope():
+            engine.model.forward(self.ctx)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         stream = torch.cuda.Stream()
         stream.wait_stream(torch.cuda.current_stream())
         with torch.cuda.stream(stream):
             with torch.cuda.graph(graph, stream=stream):
-                self.logits = engine.model.forward(self.ctx)
+                with ops.stream_scope():
+                    self.logits = engine.model.forward(self.ctx)
         torch.cuda.current_stream().wait_stream(stream)
         self.graph = graph

@@ -17,8 +17,27 @@ def dtype_code(dt) -> int:
         raise KernelError("dtype %s is not supported by the kernels (float32, bfloat16)" % dt)
 
 
+_scoped_stream = None
+
+
+class stream_scope:
+    """Looks torch's current stream up once and uses it for every launch inside the ``with`` block
+    (the lookup costs about as much as a launch).  Do not switch streams inside the block."""
+
+    def __enter__(self):
+        global _scoped_stream
+        self._outer = _scoped_stream
+        _scoped_stream = torch.cuda.current_stream().cuda_stream
+        return self
+
+    def __exit__(self, *exc):
+        global _scoped_stream
+        _scoped_stream = self._outer
+        return False
+
+
 def _stream():
-    return torch.cuda.current_stream().cuda_stream
+    return _scoped_stream if _scoped_stream is not None else torch.cuda.current_stream().cuda_stream
 
 
 def _need(cond, what):
