@@ -44,10 +44,26 @@ __device__ __forceinline__ void merge_state(float& m, float& l, float* acc, int 
                                             float mb, float lb, const float* accb) {
     const float mn = fmaxf(m, mb);
     if (mn == -INFINITY) return;                 // both empty
-    const float ca = expf(m - mn), cb = expf(mb - mn);
+    const float ca = __builtin_amdgcn_exp2f(m - mn), cb = __builtin_amdgcn_exp2f(mb - mn);   // maxima in units of log 2
     l = l * ca + lb * cb;
     for (int i = 0; i < n; ++i) acc[i] = acc[i] * ca + accb[i] * cb;
     m = mn;
+}
+
+// Sum over the LPK consecutive lanes that share a key; every one of them gets the same total.
+// Steps inside a row of 16 lanes are DPP operands of the add (no LDS round trip).
+__device__ __forceinline__ float dpp_add(float v, int) = delete;
+template <int CTRL> __device__ __forceinline__ float dpp_add(float v) {
+    return v + __int_as_float(__builtin_amdgcn_update_dpp(0, __float_as_int(v), CTRL, 0xf, 0xf, true));
+}
+template <int LPK> __device__ __forceinline__ float group_sum(float d) {
+    if (LPK >= 64) d += __shfl_xor(d, 32, kWave);
+    if (LPK >= 32) d += __shfl_xor(d, 16, kWave);
+    if (LPK >= 16) d = dpp_add<0x128>(d);        // row_ror:8      lane i <- lane i ^ 8
+    if (LPK >= 8) d = dpp_add<0x141>(d);         // row_half_mirror lane i <- lane 7 - i (of 8)
+    if (LPK >= 4) d = dpp_add<0x4E>(d);          // quad_perm [2,3,0,1]
+    if (LPK >= 2) d = dpp_add<0xB1>(d);          // quad_perm [1,0,3,2]
+    return d;
 }
 
 template <typename T, int DH, int GQ, bool STAGED>
@@ -114,20 +130,20 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
             const int hh = (h0 + j < g) ? h0 + j : g - 1;
             Vec16<T>::load(q + (size_t)t * q_stride + (size_t)(kvh * g + hh) * DH + sub * VEC, qv[j]);
 #pragma unroll
-            for (int i = 0; i < VEC; ++i) { qv[j][i] *= scale; acc[j][i] = 0.f; }
+            for (int i = 0; i < VEC; ++i) { qv[j][i] *= scale * 1.4426950408889634f; acc[j][i] = 0.f; }   // scores in units of log 2
         }
 
         // keys kb, kb + KPB, ... of one step; the next step's loads are issued before this one is used
         uint4 kr[2][kDecUnroll], vr[2][kDecUnroll];
+        // Loads are unconditional (keys beyond the share read its last key and are ignored), so the
+        // loop is straight-line code and a stage waits only for its own loads.
         auto issue = [&](int kb, uint4* kk, uint4* vv) {
 #pragma unroll
             for (int u = 0; u < kDecUnroll; ++u) {
-                const int key = kb + u * KPB;
-                if (key < hi) {
-                    const size_t off = row_of(key);
-                    kk[u] = Vec16<T>::raw(kbase + off);
-                    vv[u] = Vec16<T>::raw(vbase + off);
-                }
+                const int key = (kb + u * KPB < hi) ? kb + u * KPB : hi - 1;
+                const size_t off = row_of(key);
+                kk[u] = Vec16<T>::raw(kbase + off);
+                vv[u] = Vec16<T>::raw(vbase + off);
             }
         };
         auto consume = [&](int kb, const uint4* kk, const uint4* vv) {
@@ -136,7 +152,7 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
 #pragma unroll
             for (int u = 0; u < kDecUnroll; ++u) {
                 ok[u] = kb + u * KPB < hi;
-                if (ok[u]) Vec16<T>::unpack(kk[u], kf[u]);
+                Vec16<T>::unpack(kk[u], kf[u]);
             }
 #pragma unroll
             for (int j = 0; j < GQ; ++j) {
@@ -145,30 +161,25 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
 #pragma unroll
                 for (int u = 0; u < kDecUnroll; ++u) {
                     float d = 0.f;
-                    if (ok[u]) {
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) d += qv[j][i] * kf[u][i];
-                    }
-#pragma unroll
-                    for (int o = LPK >> 1; o > 0; o >>= 1) d += __shfl_xor(d, o, kWave);
+                    for (int i = 0; i < VEC; ++i) d += qv[j][i] * kf[u][i];
+                    d = group_sum<LPK>(d);
                     s[u] = ok[u] ? d : -INFINITY;
                     mx = fmaxf(mx, s[u]);
                 }
                 if (mx == -INFINITY) continue;     // this lane group has seen no key yet
-                const float corr = expf(m[j] - mx);
+                const float corr = __builtin_amdgcn_exp2f(m[j] - mx);
                 float lsum = l[j] * corr;
 #pragma unroll
                 for (int i = 0; i < VEC; ++i) acc[j][i] *= corr;
 #pragma unroll
                 for (int u = 0; u < kDecUnroll; ++u) {
-                    if (ok[u]) {
-                        float vf[VEC];
-                        Vec16<T>::unpack(vv[u], vf);
-                        const float p = expf(s[u] - mx);
-                        lsum += p;
+                    float vf[VEC];
+                    Vec16<T>::unpack(vv[u], vf);
+                    const float p = __builtin_amdgcn_exp2f(s[u] - mx);      // 0 for a key beyond the share
+                    lsum += p;
 #pragma unroll
-                        for (int i = 0; i < VEC; ++i) acc[j][i] += p * vf[i];
-                    }
+                    for (int i = 0; i < VEC; ++i) acc[j][i] += p * vf[i];
                 }
                 l[j] = lsum;
                 m[j] = mx;
@@ -176,12 +187,14 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
         };
         constexpr int STEP = kDecUnroll * KPB;
         const int kb0 = lo + wave * KPW + grp;
-        issue(kb0, kr[0], vr[0]);
-        for (int kb = kb0; kb < hi; kb += 2 * STEP) {
-            issue(kb + STEP, kr[1], vr[1]);
-            consume(kb, kr[0], vr[0]);
-            issue(kb + 2 * STEP, kr[0], vr[0]);
-            consume(kb + STEP, kr[1], vr[1]);
+        if (lo < hi) {                               // (block-uniform) an empty share has no key to read, not even a stand-in
+            issue(kb0, kr[0], vr[0]);
+            for (int kb = kb0; kb < hi; kb += 2 * STEP) {
+                issue(kb + STEP, kr[1], vr[1]);
+                consume(kb, kr[0], vr[0]);
+                issue(kb + 2 * STEP, kr[0], vr[0]);
+                consume(kb + STEP, kr[1], vr[1]);
+            }
         }
 
         // merge the lane groups of the wave (lanes with the same `sub`)
@@ -216,7 +229,7 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
             float a = 0.f, ll = 0.f;
             if (mm != -INFINITY) {
                 for (int w = 0; w < kDecWaves; ++w) {
-                    const float c = expf(sm_ml[w][j][0] - mm);
+                    const float c = __builtin_amdgcn_exp2f(sm_ml[w][j][0] - mm);
                     a += sm_acc[w][j][d] * c;
                     ll += sm_ml[w][j][1] * c;
                 }
@@ -224,7 +237,8 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
             const int h = kvh * g + h0 + j;
             const size_t pidx = ((size_t)n * nh + h) * nsplit + split;
             part_acc[pidx * DH + d] = a;
-            if (d == 0) { part_ml[pidx * 2] = mm; part_ml[pidx * 2 + 1] = ll; }
+            // the partial maximum leaves in natural units, as the second pass expects
+            if (d == 0) { part_ml[pidx * 2] = mm * 0.6931471805599453f; part_ml[pidx * 2 + 1] = ll; }
         }
     }
 }

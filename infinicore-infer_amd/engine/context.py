@@ -86,16 +86,13 @@ class StepContext:
         return v
 
     def decode_splits(self, n_kv_heads: int, window: int = 0) -> int:
-        """How many ways to split the keys of single-token rows.  From a sweep on MI355X: few
-        rows want about 2.25 blocks per compute unit however short the loops get; many rows want
-        about 9 per unit; a split never gets fewer than 64 keys."""
+        """How many ways to split the keys of single-token rows.  From sweeps on MI355X with a
+        cold cache: few (row, kv head) pairs want about 1.75 blocks per compute unit however short
+        the loops get; more pairs want about 3.4 per unit; a split never gets fewer than 64 keys."""
         if self.fixed_decode_splits is not None:
             return self.fixed_decode_splits
         keys = self.max_context if not window else min(self.max_context, window)
         base = max(1, self.n_decode_rows * n_kv_heads)
-        few = (9 * self.cu_count + 3) // 4
-        if base < few:
-            want = (few + base - 1) // base
-        else:
-            want = max(1, (9 * self.cu_count + base // 2) // base)
+        per_unit = 1.75 if base < 0.6 * self.cu_count else 3.4
+        want = max(1, int(per_unit * self.cu_count / base + 0.5))
         return int(max(1, min(want, max(1, keys // 64), 64)))
