@@ -299,15 +299,16 @@ IC_EXPORT int ic_attn_prefill_supported(int dtype, int dh, int page_size) {
 IC_EXPORT int ic_attn_prefill_tile_rows() { return kPfRows; }
 
 // tiles: int32 [n_tiles, 4] = (request row of block_tables, first token row, rows <= 128, position of the first row).
-IC_EXPORT int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype,
-                              const void* kcache, const void* vcache, const int* block_tables,
-                              int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
-                              int page_size, float scale, int window, hipStream_t stream) {
+// groups: 1 or 2 wave groups per query tile, 0 = chosen from the number of blocks.
+IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int out_stride, int dtype,
+                                     const void* kcache, const void* vcache, const int* block_tables,
+                                     int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
+                                     int page_size, float scale, int window, int groups, hipStream_t stream) {
     if (n_tiles <= 0) return IC_OK;
     if (!ic_attn_prefill_supported(dtype, dh, page_size)) return IC_ERR_UNSUPPORTED;
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
-    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || nh > 65535) return IC_ERR_ARG;
+    if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || nh > 65535 || groups < 0 || groups > 2) return IC_ERR_ARG;
     if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7) ||
         ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15) || ((uintptr_t)tiles & 15)) return IC_ERR_ARG;
     const float sl2 = scale * 1.4426950408889634f;
@@ -321,7 +322,7 @@ IC_EXPORT int ic_attn_prefill(const void* q, int q_stride, void* out, int out_st
             hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
         else cus = 256;
     }
-    const bool two_groups = (long long)nh * n_tiles < 6LL * cus;
+    const bool two_groups = groups ? groups == 2 : (long long)nh * n_tiles < 6LL * cus;
     dim3 grid(8 * ((nh + 7) / 8) * n_tiles);
 #define IC_PF_LAUNCH(DD, ST, GG)                                                                                   \
     hipLaunchKernelGGL((attn_prefill_mfma_kernel<DD, ST, GG>), grid, dim3(256 * GG), 0, stream, (const uint16_t*)q, \
@@ -335,4 +336,12 @@ IC_EXPORT int ic_attn_prefill(const void* q, int q_stride, void* out, int out_st
     else
         return IC_ERR_UNSUPPORTED;
     return ic_launch_status();
+}
+
+IC_EXPORT int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype,
+                              const void* kcache, const void* vcache, const int* block_tables,
+                              int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
+                              int page_size, float scale, int window, hipStream_t stream) {
+    return ic_attn_prefill_groups(q, q_stride, out, out_stride, dtype, kcache, vcache, block_tables, bt_stride, tiles,
+                                  n_tiles, nh, nkvh, dh, page_size, scale, window, 0, stream);
 }

@@ -41,6 +41,8 @@ int ic_attn_decode(const void* q, int q_stride, void* out, int out_stride, int d
 int ic_attn_prefill_supported(int dtype, int dh, int page_size);
 int ic_attn_prefill_tile_rows();
 int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, hipStream_t stream);
+// The same with the number of wave groups per query tile given: 2 halves the longest tile's walk over the keys (few blocks), 1 keeps more blocks resident (many blocks), 0 chooses.
+int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, hipStream_t stream);
 
 // ---- gemm.hip ---------------------------------------------------------------------------------------
 // A norm y = x * rsqrt(mean(x^2) + eps) * w between two products of M <= 16 rows can be split over them: the

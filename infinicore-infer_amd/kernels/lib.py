@@ -53,6 +53,7 @@ _SIGNATURES = {
     "ic_attn_prefill_supported": [_I, _I, _I],
     "ic_attn_prefill_tile_rows": [],
     "ic_attn_prefill": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _P],
+    "ic_attn_prefill_groups": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],

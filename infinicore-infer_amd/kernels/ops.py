@@ -215,16 +215,18 @@ def attention_prefill_tile_rows() -> int:
 
 
 def attention_prefill(q, out, kcache, vcache, block_tables, tiles, n_tiles, n_heads, n_kv_heads, head_dim,
-                      page_size, scale: float, window: int = 0):
+                      page_size, scale: float, window: int = 0, groups: int = 0):
     """Matrix-core attention of prompt portions.  tiles: int32 [n, 4] rows of
-    (request row in block_tables, first token row, rows <= tile_rows, first position)."""
+    (request row in block_tables, first token row, rows <= tile_rows, first position).
+    groups: wave groups per query tile (1 or 2); 0 lets the kernel choose from the number of blocks."""
+    _need(groups in (0, 1, 2), "attention_prefill: groups must be 0, 1 or 2")
     _attn_common(q, out, kcache, vcache, block_tables, n_heads, n_kv_heads, head_dim, page_size)
     _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.dim() == 2 and tiles.shape[1] == 4
           and tiles.shape[0] >= n_tiles, "attention_prefill: tiles must be int32 [n, 4]")
-    check(get_lib().ic_attn_prefill(
+    check(get_lib().ic_attn_prefill_groups(
         q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype), kcache.data_ptr(),
         vcache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), tiles.data_ptr(), n_tiles,
-        n_heads, n_kv_heads, head_dim, page_size, float(scale), int(window or 0), _stream()),
+        n_heads, n_kv_heads, head_dim, page_size, float(scale), int(window or 0), int(groups), _stream()),
         "attention_prefill")
 
 

@@ -155,8 +155,9 @@ def test_rope_kv_write(dtype, nh, nkvh, dh, rot, page):
         _close(got[:, :nh][..., perm], adj, dtype)
 
 
-def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl):
-    """lens: list of (past, new) per request.  Returns (got, want) [T, nh*dh]."""
+def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_width=0, groups=0):
+    """lens: list of (past, new) per request.  Returns (got, want) [T, nh*dh].  table_width pads
+    the block tables with unused columns; groups is passed to the prompt-portion kernel."""
     ops = _ops()
     g = torch.Generator().manual_seed(seed)
     scale = 1.0 / math.sqrt(dh)
@@ -175,7 +176,7 @@ def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl):
         qs.append(q.reshape(new, nh * dh))
         token_req += [r] * new
         positions += list(range(past, t))
-    maxb = max(len(b) for b in tables)
+    maxb = max(max(len(b) for b in tables), table_width)
     bt = torch.zeros(len(lens), maxb, dtype=torch.int32)
     for r, b in enumerate(tables):
         bt[r, :len(b)] = b
@@ -203,7 +204,7 @@ def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl):
                 tiles += [r, row0 + o, min(rows, new - o), past + o]
             row0 += new
         tl = torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 4)
-        ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0)
+        ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0, groups)
     return out, torch.cat(want)
 
 
@@ -230,10 +231,28 @@ def test_attention_decode(dtype, nh, nkvh, dh, page, window):
 @pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (3, 1, 64, 32), (4, 2, 128, 16),
                                               (4, 4, 128, 64)])
 @pytest.mark.parametrize("window", [None, 100])
-def test_attention_prefill_mfma(nh, nkvh, dh, page, window):
+@pytest.mark.parametrize("groups", [1, 2])
+def test_attention_prefill_mfma(nh, nkvh, dh, page, window, groups):
     lens = [(0, 2), (0, 129), (130, 64), (64, 33), (15, 2), (257, 300), (5, 128)]
-    got, want = _attention_case(torch.bfloat16, nh, nkvh, dh, page, lens, window, 13, "prefill")
+    got, want = _attention_case(torch.bfloat16, nh, nkvh, dh, page, lens, window, 13, "prefill", groups=groups)
     _close(got, want, torch.bfloat16, factor=3)
+
+
+@pytest.mark.parametrize("impl,dtype,nh,nkvh,dh", [("decode", torch.bfloat16, 6, 6, 64), ("decode", torch.float32, 4, 4, 128),
+                                                     ("decode", torch.bfloat16, 6, 2, 64), ("decode", torch.float32, 6, 2, 64),
+                                                     ("decode", torch.bfloat16, 16, 1, 128),
+                                                     ("prefill1", torch.bfloat16, 6, 2, 64), ("prefill2", torch.bfloat16, 6, 2, 64),
+                                                     ("prefill1", torch.bfloat16, 4, 4, 128), ("prefill2", torch.bfloat16, 4, 2, 128)])
+def test_attention_with_block_tables_too_wide_to_stage(impl, dtype, nh, nkvh, dh):
+    """Block tables wider than the page-id staging area: the kernels read page ids from memory."""
+    if impl == "decode":
+        lens = [(0, 1), (63, 1), (700, 1), (255, 1)]
+        got, want = _attention_case(dtype, nh, nkvh, dh, 16, lens, 100 if nh == 6 else None, 15, "decode", table_width=2100)
+    else:
+        lens = [(0, 129), (130, 64), (257, 300)]
+        got, want = _attention_case(dtype, nh, nkvh, dh, 16, lens, None, 16, "prefill", table_width=2100,
+                                    groups=int(impl[-1]))
+    _close(got, want, dtype, factor=3)
 
 
 def test_attention_special_cases():
