@@ -137,6 +137,7 @@ def main():
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
     ap.add_argument("--no-tune", action="store_true", help="keep the library's default kernel choice for prefill products")
     ap.add_argument("--batch", type=int, default=BATCH, help="batch of the headline run (for profiling other points)")
+    ap.add_argument("--eager", action="store_true", help="decode without HIP graphs (so that a profiler's counters attribute to kernels)")
     args = ap.parse_args()
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
@@ -151,6 +152,8 @@ def main():
     engine, conf = build_engine(args.layers, per_req * max(batches), max(batches) + 1, args.page_size)
     weight_bytes, kv_per_tok, prefill_flops = model_numbers(conf)
     vocab = conf.vocab_size
+    if args.eager:
+        engine.use_graphs = False
 
     if not args.no_tune:
         engine.tune_library_products([PROMPT])      # the library's kernel choice for 2,048-row products
@@ -179,6 +182,7 @@ def main():
             "global_batch": BATCH, "seq_len": PROMPT, "context_mean": round(ctx, 1), "generated": args.steps,
             "page_size": args.page_size, "tied_embeddings": bool(MODEL.get("tie_word_embeddings", True)), "parallelism": "single-gpu",
             "sampling": "greedy on device", "library_gemm": "default" if args.no_tune else "tuned for prefill",
+            "decode_launch": "eager" if args.eager else "hip graph",
         },
         "prefill": {"value": round(PROMPT / t_pf, 1), "tokens": PROMPT, "ms": round(t_pf * 1e3, 3),
                     "frac": round(pf_flops / t_pf / (PEAK_TFLOPS["bf16"] * 1e12), 4)},
