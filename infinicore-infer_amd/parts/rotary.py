@@ -90,9 +90,8 @@ class Rotary(PositionEncoding):
 
 @register_part("position_encoding", "none")
 class NoPositionEncoding(PositionEncoding):
-    graph_safe = True
-
     """No rotation: only the cache write."""
+    graph_safe = True
 
     def __init__(self, name, runtime, **_):
         super().__init__(name, runtime)

@@ -371,3 +371,156 @@ def test_toy_architecture_with_a_stateful_mixer(tmp_path_factory):
     eng.step([StepEntry("w", requests["t2"][:100], [])])
     wg = [i for i, g in enumerate(eng.groups) if g.kind == "window"][0]
     assert eng.cache.free_pages(wg) > eng.cache.free_pages(1 - wg)
+
+
+# ---------------------------------------------------------------------------
+# a second toy architecture: a feed-forward with routing and another position encoding
+# ---------------------------------------------------------------------------
+def _register_toy_routed():
+    from infinicore_infer_amd.config import LayerSpec, ModelSpec, PartSpec, default_schedule, register_architecture
+    from infinicore_infer_amd.parts import FeedForward, PositionEncoding, register_part
+    from infinicore_infer_amd.parts.rotary import NoPositionEncoding
+    from infinicore_infer_amd.weights import WeightSpec
+
+    @register_part("feed_forward", "toy_top1_experts")
+    class Top1Experts(FeedForward):
+        """Router logits in float32, the best expert per token, experts = up, GELU, down."""
+
+        def __init__(self, name, runtime, hidden_size, inner_size, num_experts):
+            super().__init__(name, runtime)
+            self.d, self.di, self.ne = hidden_size, inner_size, num_experts
+
+        def weight_specs(self):
+            n = self.name
+            s = {n + "router.weight": WeightSpec((self.ne, self.d))}
+            for i in range(self.ne):
+                s[n + "experts.%d.up.weight" % i] = WeightSpec((self.di, self.d))
+                s[n + "experts.%d.down.weight" % i] = WeightSpec((self.d, self.di))
+            return s
+
+        def load_weights(self, tensors):
+            n = self.name
+            self.router = tensors[n + "router.weight"]
+            self.up = [tensors[n + "experts.%d.up.weight" % i] for i in range(self.ne)]
+            self.down = [tensors[n + "experts.%d.down.weight" % i] for i in range(self.ne)]
+
+        def forward(self, h, ctx):
+            choice = (h.float() @ self.router.float().t()).argmax(-1)
+            y = ctx.ws.buffer("toy_ffn_out", tuple(h.shape), self.runtime.dtype)
+            for i in range(self.ne):
+                rows = (choice == i).nonzero().flatten()
+                if rows.numel():
+                    a = torch.nn.functional.gelu(h[rows] @ self.up[i].t())
+                    y[rows] = a @ self.down[i].t()
+            return y
+
+    @register_part("position_encoding", "toy_adjacent_pairs")
+    class AdjacentPairs(PositionEncoding):
+        """Rotates pairs (2j, 2j + 1) of q and k by pos * base^-j, then stores k and v as they are."""
+
+        def __init__(self, name, runtime, head_dim, base):
+            super().__init__(name, runtime)
+            self.dh, self.base = head_dim, float(base)
+            self.store = NoPositionEncoding(name, runtime)
+
+        def rotate_and_store(self, qkv, ctx, cache, n_heads, n_kv_heads, head_dim):
+            T = qkv.shape[0]
+            j = torch.arange(head_dim // 2, device=qkv.device, dtype=torch.float32)
+            ang = ctx.positions.float()[:, None] * self.base ** (-j)[None, :]
+            c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+            x = qkv[:, :(n_heads + n_kv_heads) * head_dim].reshape(T, n_heads + n_kv_heads, head_dim // 2, 2).float()
+            a, b = x[..., 0], x[..., 1]
+            rot = torch.stack([a * c - b * s, a * s + b * c], -1).reshape(T, -1)
+            qkv[:, :(n_heads + n_kv_heads) * head_dim] = rot.to(qkv.dtype)
+            self.store.rotate_and_store(qkv, ctx, cache, n_heads, n_kv_heads, head_dim)
+
+    class RoutedConfig:
+        def __init__(self, cfg):
+            self.cfg = cfg
+
+        @classmethod
+        def from_dict(cls, cfg, **kw):
+            return cls(cfg)
+
+        def model_spec(self):
+            c = self.cfg
+            d, nh, dh = c["hidden"], c["heads"], c["head_dim"]
+            pe = PartSpec("toy_adjacent_pairs", "", {"head_dim": dh, "base": c["base"]})
+            norm = lambda p: PartSpec("rmsnorm", p, {"size": d, "eps": 1e-6})
+            layers = []
+            for i in range(c["layers"]):
+                p = "blocks.%d." % i
+                ffn = PartSpec("toy_top1_experts", p + "moe.", {"hidden_size": d, "inner_size": c["inner"], "num_experts": c["experts"]}) \
+                    if i % 2 == 0 else PartSpec("swiglu", p + "mlp.", {"hidden_size": d, "intermediate_size": c["inner"]})
+                att = PartSpec("attention", p + "att.", {"hidden_size": d, "num_heads": nh, "num_kv_heads": nh, "head_dim": dh,
+                                                         "softmax_scale": dh ** -0.5, "position_encoding": pe})
+                layers.append(LayerSpec(PartSpec("prenorm_residual", p, {"residual_scale": 1.0}), att, norm(p + "n1."),
+                                        ffn, norm(p + "n2.")))
+            return ModelSpec("toy-routed", c["vocab"], d, c["max_pos"],
+                             PartSpec("embedding", "emb.", {"vocab_size": c["vocab"], "hidden_size": d, "scale": 1.0}),
+                             layers, default_schedule(len(layers)), norm("final."),
+                             PartSpec("lm_head", "head.", {"vocab_size": c["vocab"], "hidden_size": d, "logit_scale": 1.0}))
+
+    register_architecture(["toy-routed-arch"], RoutedConfig)
+
+
+def _toy_routed_plain(model, cfg, tokens):
+    T, nh, dh = len(tokens), cfg["heads"], cfg["head_dim"]
+    cpu = lambda t: t.detach().cpu().double()
+    j = torch.arange(dh // 2, dtype=torch.float64)
+    ang = torch.arange(T, dtype=torch.float64)[:, None] * cfg["base"] ** (-j)[None, :]
+    c, s = ang.cos()[:, None, :], ang.sin()[:, None, :]
+
+    def rot(x):                                     # [T, heads, dh], adjacent pairs
+        a, b = x[..., 0::2], x[..., 1::2]
+        return torch.stack([a * c - b * s, a * s + b * c], -1).reshape(x.shape)
+
+    x = P.plain_embedding(cpu(model.embedding.table), tokens, 1.0)
+    for blk in model.layers:
+        h = P.plain_rmsnorm(x, cpu(blk.mixer_norm.weight), 1e-6)
+        qkv = P.plain_linear(h, cpu(blk.mixer.w_qkv)).reshape(T, 3 * nh, dh)
+        q, k, v = rot(qkv[:, :nh]), rot(qkv[:, nh:2 * nh]), qkv[:, 2 * nh:]
+        a = P.plain_attention(q, k, v, dh ** -0.5, 0, None).reshape(T, nh * dh)
+        x = x + P.plain_linear(a, cpu(blk.mixer.w_o))
+        h = P.plain_rmsnorm(x, cpu(blk.feed_forward_norm.weight), 1e-6)
+        f = blk.feed_forward
+        if hasattr(f, "router"):
+            choice = P.plain_linear(h, cpu(f.router)).argmax(-1)
+            y = torch.zeros_like(h)
+            for t in range(T):
+                i = int(choice[t])
+                y[t] = P.plain_linear(torch.nn.functional.gelu(P.plain_linear(h[t:t + 1], cpu(f.up[i]))), cpu(f.down[i]))[0]
+        else:
+            gu = P.plain_linear(h, cpu(f.w_gate_up))
+            di = gu.shape[1] // 2
+            y = P.plain_linear(P.plain_swiglu(gu[:, :di], gu[:, di:]), cpu(f.w_down))
+        x = x + y
+    return P.plain_linear(P.plain_rmsnorm(x, cpu(model.final_norm.weight), 1e-6), cpu(model.head.weight))
+
+
+def test_toy_architecture_with_routed_experts_and_another_position_encoding():
+    """A feed-forward with routing and a position encoding of its own, both defined here, chosen
+    layer by layer beside the package's parts, registered, built and stepped through the engine."""
+    from infinicore_infer_amd.config import config_from_dict
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.parts import Runtime, build_model
+    from infinicore_infer_amd.weights import init_random_weights
+    _register_toy_routed()
+    cfg = {"model_type": "toy-routed-arch", "vocab": 61, "hidden": 40, "heads": 5, "head_dim": 16, "inner": 56,
+           "experts": 3, "layers": 3, "base": 50.0, "max_pos": 128}
+    model = build_model(config_from_dict(cfg).model_spec(), Runtime(torch.float32, DEV))
+    init_random_weights(model, seed=5, std=0.2, norm_std=0.1, tie=False)
+    requests = {"m%d" % i: H.random_tokens(61, n, 60 + i) for i, n in enumerate([50, 17, 90])}
+    ref = {rid: _toy_routed_plain(model, cfg, toks) for rid, toks in requests.items()}
+    used = set()
+    for blk in model.layers:
+        if hasattr(blk.feed_forward, "router"):
+            used.add(type(blk.feed_forward).__name__)
+    assert used == {"Top1Experts"}
+    for maker in (H.trace_whole, H.trace_chunks, H.trace_mixed):
+        steps, max_tokens = maker(requests)
+        eng = Engine(model, max_tokens=max_tokens, page_size=16, max_requests=4)
+        assert not eng.use_graphs                      # parts that do not declare graph_safe keep the engine eager
+        got = H.run_trace(eng, steps)
+        H.compare(got, ref, 2e-4, "toy routed %s" % maker.__name__)
+        eng.cache.check_invariants()
