@@ -75,6 +75,16 @@ int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, in
 int ic_gemm_qkv_rope_supported(int dtype, int dh);
 int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc, const int* positions, const int* slots, const float* cos_t, const float* sin_t, void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size, const IcRowFactor* row_factor, hipStream_t stream);
 
+// ---- matmul_library.hip ------------------------------------------------------------------------------
+// The library (hipBLASLt) matrix product for many rows: C[M, N] = alpha * A[M, K] W[N, K]^T, bfloat16 operands with a
+// bfloat16 or float32 result, or all float32 (true float32).  Descriptors and the algorithm are kept per shape.
+// Returns -3 when the library refuses a call and -4 when it proposes no algorithm.  These two allocate host-side
+// descriptors at the first call of a shape; workspace is device memory passed in by the caller.
+int ic_matmul_supported(int a_dtype, int c_dtype);
+int ic_matmul(const void* A, int a_dtype, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, void* workspace, long long workspace_bytes, hipStream_t stream);
+// Times the algorithms the library proposes for this shape and keeps the fastest; returns how many were tried.
+int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, void* workspace, long long workspace_bytes, int reps, hipStream_t stream);
+
 // ---- sampling.hip -----------------------------------------------------------------------------------
 // Greedy choice per row; scratch_val / scratch_idx: 64 * n_rows elements.
 int ic_argmax(const float* logits, long long row_stride, int n_rows, int V, float* scratch_val, int* scratch_idx, int* out, hipStream_t stream);

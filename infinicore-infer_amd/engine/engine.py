@@ -329,21 +329,14 @@ class Engine:
         return g.logits
 
     # ---- library products ----------------------------------------------------------------------------
-    def tune_library_products(self, token_counts: Sequence[int], max_ms_per_shape: int = 300) -> None:
-        """Let the library pick its fastest matrix-product kernel for prompt portions of the given
-        token counts (PyTorch's tunable-op mechanism over hipBLASLt and rocBLAS): one dummy step per
-        count is run with tuning on, then tuning is switched off again, so other shapes keep the
-        library's default choice and cost nothing.  Optional; results live for this process."""
-        import torch.cuda.tunable as tunable
-        tunable.enable(True)
-        tunable.tuning_enable(True)
-        tunable.set_max_tuning_duration(int(max_ms_per_shape))
-        if hasattr(tunable, "write_file_on_exit"):
-            tunable.write_file_on_exit(False)
-        else:                                     # keep the results file out of the working directory
-            import os
-            import tempfile
-            tunable.set_filename(os.path.join(tempfile.gettempdir(), "infinicore_infer_amd-tunable-%d.csv" % os.getpid()))
+    def tune_library_products(self, token_counts: Sequence[int]) -> None:
+        """Let the library's matrix products for prompt portions of the given token counts use their
+        fastest algorithm: one dummy step per count is run in which every library product first times
+        the algorithms the library proposes for its shape on the device and keeps the best.  Other
+        shapes keep the library's first choice and cost nothing.  Optional; results live for this
+        process."""
+        from ..parts import linear as _linear
+        _linear.TUNE_LIBRARY = True
         try:
             for n in token_counts:
                 rid = ("tune", n)
@@ -351,7 +344,7 @@ class Engine:
                 self.free(rid)
             torch.cuda.synchronize()
         finally:
-            tunable.tuning_enable(False)
+            _linear.TUNE_LIBRARY = False
 
     # ---- sampling --------------------------------------------------------------------------------------
     def sample(self, logits, temperature=None, top_k=None, top_p=None, uniform=None) -> List[int]:

@@ -23,6 +23,7 @@ HIPCC_FLAGS = [
     "-Xclang", "-target-feature", "-Xclang", "-packed-fp32-ops",
     "-Wno-unused-command-line-argument",
 ]
+LINK_LIBS = ["-lhipblaslt"]          # the library matrix product for many rows (matmul_library.hip)
 
 
 class BuildError(RuntimeError):
@@ -35,7 +36,7 @@ def sources():
 
 def source_hash() -> str:
     h = hashlib.sha1()
-    h.update(" ".join(HIPCC_FLAGS).encode())
+    h.update(" ".join(HIPCC_FLAGS + LINK_LIBS).encode())
     for f in sorted(os.listdir(CSRC)):
         if f.endswith((".hip", ".h")):
             h.update(f.encode())
@@ -111,7 +112,7 @@ def build(force: bool = False, verbose: bool = True) -> str:
     with ThreadPoolExecutor(max_workers=workers) as ex:
         objs = list(ex.map(compile_one, srcs))
     tmp = os.path.join(out_dir, ".%s.%d.tmp" % (name, os.getpid()))
-    cmd = [hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs
+    cmd = [hipcc, "--offload-arch=" + ARCH, "-shared", "-fPIC", "-o", tmp] + objs + LINK_LIBS
     r = subprocess.run(cmd, stdout=subprocess.PIPE, stderr=subprocess.STDOUT, text=True)
     if r.returncode != 0:
         raise BuildError("link failed:\n%s" % r.stdout)

@@ -329,6 +329,59 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
     return out
 
 
+_matmul_workspace = {}
+MATMUL_WORKSPACE_BYTES = 64 << 20
+
+
+def _workspace(device):
+    ws = _matmul_workspace.get(device)
+    if ws is None:
+        ws = _matmul_workspace[device] = torch.empty(MATMUL_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+    return ws
+
+
+class NoLibraryAlgorithm(KernelError):
+    """The library proposes no algorithm for a product."""
+
+
+def _matmul_args(a, w, out, what):
+    _dev(a, w, out)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(w.shape[1] == K and tuple(out.shape) == (M, N), what + ": shape mismatch")
+    _need(a.dtype == w.dtype and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, what + ": layout")
+    _need(bool(get_lib().ic_matmul_supported(dtype_code(a.dtype), dtype_code(out.dtype))), what + ": unsupported types")
+    return M, N, K
+
+
+def matmul_library(a, w, out, alpha: float = 1.0):
+    """out[M, N] = alpha * a[M, K] @ w[N, K]^T through the library (hipBLASLt), any number of rows.
+    bfloat16 operands with a bfloat16 or float32 result, or all float32."""
+    M, N, K = _matmul_args(a, w, out, "matmul_library")
+    ws = _workspace(a.device)
+    st = get_lib().ic_matmul(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), out.data_ptr(), dtype_code(out.dtype),
+                             M, N, K, a.stride(0), w.stride(0), out.stride(0), float(alpha), ws.data_ptr(), ws.numel(),
+                             _stream())
+    if st == -4:
+        raise NoLibraryAlgorithm("matmul_library: no algorithm for %d x %d x %d" % (M, N, K))
+    if st == -3:
+        raise KernelError("matmul_library: the library refused the product %d x %d x %d" % (M, N, K))
+    check(st, "matmul_library")
+    return out
+
+
+def matmul_library_tune(a, w, out, reps: int = 5) -> int:
+    """Times the library's algorithms for this product's shape and keeps the fastest; returns how many it tried."""
+    M, N, K = _matmul_args(a, w, out, "matmul_library_tune")
+    ws = _workspace(a.device)
+    n = get_lib().ic_matmul_tune(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), out.data_ptr(), dtype_code(out.dtype),
+                                 M, N, K, a.stride(0), w.stride(0), out.stride(0), ws.data_ptr(), ws.numel(), int(reps),
+                                 _stream())
+    if n < 0:
+        raise KernelError("matmul_library_tune failed with %d for %d x %d x %d" % (n, M, N, K))
+    return n
+
+
 def gemm_qkv_rope_supported(dtype, head_dim: int) -> bool:
     try:
         return bool(get_lib().ic_gemm_qkv_rope_supported(dtype_code(dtype), head_dim))

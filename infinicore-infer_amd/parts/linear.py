@@ -16,25 +16,30 @@ torch.backends.cuda.matmul.allow_tf32 = False
 torch.backends.cudnn.allow_tf32 = False
 
 FEW_ROWS = 16          # up to here the package's own kernel beats the library on MI355X
-_mm_out_dtype_ok = None
+TUNE_LIBRARY = False   # while True, every library product times the library's algorithms for its shape first
+_tuned = set()
 
 
-def _library_mm_f32_out(x, w, out):
-    """bfloat16 operands, float32 result: the library's mixed-output product when it has one."""
-    global _mm_out_dtype_ok
-    if _mm_out_dtype_ok is None:
-        try:
-            torch.mm(x[:1], w[:1].t(), out_dtype=torch.float32)
-            _mm_out_dtype_ok = True
-        except Exception:
-            _mm_out_dtype_ok = False
-    if _mm_out_dtype_ok:
-        try:
-            torch.mm(x, w.t(), out_dtype=torch.float32, out=out)
-        except (TypeError, RuntimeError):
-            out.copy_(torch.mm(x, w.t(), out_dtype=torch.float32))
-    else:
-        ops.gemm_nt(x, w, out)
+def _library(x, w, out, alpha: float = 1.0):
+    """out = alpha * x w^T through the library, as the reference does for every product
+    (inference_context.cpp:59-79): hipBLASLt called directly, torch's routine if it has no
+    algorithm for the shape."""
+    if TUNE_LIBRARY:
+        key = (x.dtype, out.dtype, x.shape[0], w.shape[0], w.shape[1], x.stride(0), w.stride(0), out.stride(0))
+        if key not in _tuned:
+            _tuned.add(key)
+            try:
+                ops.matmul_library_tune(x, w, out)
+            except ops.KernelError:
+                pass
+    try:
+        return ops.matmul_library(x, w, out, alpha)
+    except ops.NoLibraryAlgorithm:
+        if out.dtype == x.dtype:
+            torch.mm(x, w.t(), out=out)
+        else:
+            out.copy_(torch.mm(x.to(out.dtype), w.to(out.dtype).t()))
+        return out.mul_(alpha) if alpha != 1.0 else out
 
 
 def own_kernel_applies(M, x_dtype, w_dtype, out_dtype, impl: str) -> bool:
@@ -50,25 +55,15 @@ def linear(x, w, out, impl: str = "auto", alpha: float = 1.0):
         if own_kernel_applies(x.shape[0], x.dtype, w.dtype, out.dtype, impl):
             return ops.gemm_nt(x.values, w, out, alpha=alpha, row_factor=x.row_factor())
         x = x.materialize()
-    if alpha != 1.0:
-        if own_kernel_applies(x.shape[0], x.dtype, w.dtype, out.dtype, impl):
-            return ops.gemm_nt(x, w, out, alpha=alpha)
-        linear(x, w, out, impl)
-        return out.mul_(alpha)
     if w.dtype != x.dtype:
         # a matrix stored in 32-bit stays so: compute this product in float32
-        tmp = torch.mm(x.to(torch.float32), w.to(torch.float32).t())
+        tmp = torch.empty(out.shape, dtype=torch.float32, device=out.device)
+        _library(x.to(torch.float32), w.to(torch.float32), tmp, alpha)
         out.copy_(tmp)
         return out
-    M = x.shape[0]
-    if x.dtype == torch.bfloat16:
-        if (impl == "auto" and M <= FEW_ROWS) and ops.gemm_nt_supported(x.dtype, w.dtype, out.dtype):
-            return ops.gemm_nt(x, w, out)
-        if out.dtype == torch.float32:
-            _library_mm_f32_out(x, w, out)
-            return out
-    torch.mm(x, w.t(), out=out)
-    return out
+    if own_kernel_applies(x.shape[0], x.dtype, w.dtype, out.dtype, impl):
+        return ops.gemm_nt(x, w, out, alpha=alpha)
+    return _library(x, w, out, alpha)
 
 
 def linear_tail(x, w, tail, ws, name: str, impl: str = "auto"):
