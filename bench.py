@@ -156,7 +156,8 @@ def main():
         engine.use_graphs = False
 
     if not args.no_tune:
-        engine.tune_library_products([PROMPT])      # the library's kernel choice for 2,048-row products
+        # the library's algorithm choice for the products of the prefill and of decoding at batches beyond 16
+        engine.tune_library_products([PROMPT] + [b for b in batches if b > 16])
     g = torch.Generator().manual_seed(123)
     ptoks = torch.randint(0, vocab, (PROMPT,), generator=g).tolist()
     t_pf = time_prefill(engine, ptoks)
@@ -181,7 +182,7 @@ def main():
             "head_dim": conf.head_dim, "intermediate": conf.intermediate_size, "vocab": conf.vocab_size,
             "global_batch": BATCH, "seq_len": PROMPT, "context_mean": round(ctx, 1), "generated": args.steps,
             "page_size": args.page_size, "tied_embeddings": bool(MODEL.get("tie_word_embeddings", True)), "parallelism": "single-gpu",
-            "sampling": "greedy on device", "library_gemm": "default" if args.no_tune else "tuned for prefill",
+            "sampling": "greedy on device", "library_gemm": "default" if args.no_tune else "algorithms timed per shape",
             "decode_launch": "eager" if args.eager else "hip graph",
         },
         "prefill": {"value": round(PROMPT / t_pf, 1), "tokens": PROMPT, "ms": round(t_pf * 1e3, 3),
