@@ -77,7 +77,7 @@ def model_numbers(conf):
     return weight_bytes, kv_bytes_per_token, prefill_flops
 
 
-def time_prefill(engine, tokens, reps=3):
+def time_prefill(engine, tokens, reps=6):
     from infinicore_infer_amd.engine import StepEntry
     best = None
     for i in range(reps + 1):

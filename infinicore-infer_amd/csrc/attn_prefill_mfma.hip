@@ -1,7 +1,7 @@
 // Attention of prompt portions over the paged cache on the matrix cores
 // (bfloat16 operands, float32 accumulation and softmax).
 //
-// Grid (8 * ceil(heads / 8) * query tiles), 256 * GROUPS threads, dealt to the XCDs head by head.  A tile is up to 128
+// Grid (heads * query tiles), tile-major, 256 * GROUPS threads.  A tile is up to 128
 // consecutive tokens of one request; wave w of a group owns rows 32w..32w+31.  With GROUPS == 2
 // the two groups take the even and the odd key tiles of 64 and are merged through LDS at the
 // end: the longest query tile of a prompt, which sets the kernel's time when there are few
@@ -61,12 +61,13 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
 
     __shared__ int pages[kPfMaxPages];
 
-    // Blocks are dealt to the 8 XCDs in turn (each has an L2 of its own): block b runs on XCD
-    // b % 8.  All tiles of a head are given to one XCD, so that head's keys stay in that L2.
-    const int xcd = blockIdx.x & 7, seq = blockIdx.x >> 3;
-    const int h = xcd + 8 * (seq / n_tiles);
-    if (h >= nh) return;
-    const int4 tile = tiles[seq % n_tiles];
+    // Blocks start in index order and the host lists the tiles longest first: tile-major order (all heads
+    // of the longest tile, then of the next one) therefore starts the long walks first everywhere, and since
+    // blocks are dealt to the 8 XCDs in turn (block b runs on XCD b % 8) every XCD gets an equal share of
+    // every length.  A head's tiles then meet on few XCDs (two of them with 36 heads), so its keys still
+    // stay in those L2s.
+    const int h = blockIdx.x % nh;
+    const int4 tile = tiles[blockIdx.x / nh];
     const int req = tile.x, row0 = tile.y, n_rows = tile.z, pos0 = tile.w;
     const int kvh = h / (nh / nkvh);
     const int* bt = block_tables + (size_t)req * bt_stride;
@@ -313,7 +314,7 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
         ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15) || ((uintptr_t)tiles & 15)) return IC_ERR_ARG;
     const float sl2 = scale * 1.4426950408889634f;
     const bool staged = bt_stride <= kPfMaxPages;       // a block never needs more page ids than a request has
-    // Few blocks (up to 6 per compute unit, measured): the longest tile's walk over the keys sets the
+    // Few blocks (under 2.75 per compute unit, measured): the longest tile's walk over the keys sets the
     // time, so two wave groups share it.  Many blocks: one group, more blocks resident.
     static int cus = 0;                                 // compute units of the device, asked once
     if (cus == 0) {
@@ -322,8 +323,8 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
             hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
         else cus = 256;
     }
-    const bool two_groups = groups ? groups == 2 : (long long)nh * n_tiles < 6LL * cus;
-    dim3 grid(8 * ((nh + 7) / 8) * n_tiles);
+    const bool two_groups = groups ? groups == 2 : 4LL * nh * n_tiles < 11LL * cus;
+    dim3 grid((unsigned)nh * (unsigned)n_tiles);
 #define IC_PF_LAUNCH(DD, ST, GG)                                                                                   \
     hipLaunchKernelGGL((attn_prefill_mfma_kernel<DD, ST, GG>), grid, dim3(256 * GG), 0, stream, (const uint16_t*)q, \
                        q_stride, (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
