@@ -74,7 +74,8 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
                          const int* __restrict__ tok_list, const int* __restrict__ token_req,
                          const int* __restrict__ positions,
                          float* __restrict__ part_acc, float* __restrict__ part_ml,
-                         int nh, int nkvh, int page_size, float scale, int window, int nsplit) {
+                         int nh, int nkvh, int page_size, float scale, int window, int nsplit,
+                         T* __restrict__ final_out, int out_stride) {
     constexpr int VEC = Vec16<T>::N;
     constexpr int LPK = DH / VEC;                 // lanes per key
     constexpr int KPW = 64 / LPK;                 // keys per wave per step
@@ -235,6 +236,10 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
                 }
             }
             const int h = kvh * g + h0 + j;
+            if (final_out) {                        // a single split: this is the result, no second pass
+                final_out[(size_t)t * out_stride + (size_t)h * DH + d] = from_f32<T>(a / ll);
+                continue;
+            }
             const size_t pidx = ((size_t)n * nh + h) * nsplit + split;
             part_acc[pidx * DH + d] = a;
             // the partial maximum leaves in natural units, as the second pass expects
@@ -301,7 +306,8 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
                        const int* __restrict__ tok_list, const int* __restrict__ token_req,
                        const int* __restrict__ positions,
                        float* __restrict__ part_acc, float* __restrict__ part_ml,
-                       int nh, int nkvh, int page_size, float scale, int window, int nsplit) {
+                       int nh, int nkvh, int page_size, float scale, int window, int nsplit,
+                       uint16_t* __restrict__ final_out, int out_stride) {
     constexpr int NC = DH / 32;                    // 32-dim chunks of the score product
     constexpr int ND = DH / 16;                    // 16-dim chunks of the output
     constexpr int VS = DH + 8;                     // LDS row stride of a V tile (elements)
@@ -479,6 +485,10 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
                 }
             }
             const int h = kvh * g + h0 + j;
+            if (final_out) {                        // a single split: this is the result, no second pass
+                final_out[(size_t)t * out_stride + (size_t)h * DH + d] = f32_to_bf16_bits(a / ll);
+                continue;
+            }
             const size_t pidx = ((size_t)n * nh + h) * nsplit + split;
             part_acc[pidx * DH + d] = a;
             if (d == 0) { part_ml[pidx * 2] = mm; part_ml[pidx * 2 + 1] = ll; }
@@ -495,10 +505,11 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
                          hipStream_t stream) {
     dim3 grid(nsplit, nkvh, n_tok), block(kDecThreads);
     const bool staged = bt_stride <= kDecMaxPages;      // a block never needs more page ids than a request has
+    void* direct = (nsplit == 1) ? out : nullptr;       // one split writes the result itself
 #define IC_DEC_LAUNCH(KERNEL, TQ)                                                                           \
     hipLaunchKernelGGL(KERNEL, grid, block, 0, stream, (const TQ*)q, q_stride, (const TQ*)kcache,           \
                        (const TQ*)vcache, block_tables, bt_stride, tok_list, token_req, positions, part_acc, \
-                       part_ml, nh, nkvh, page_size, scale, window, nsplit)
+                       part_ml, nh, nkvh, page_size, scale, window, nsplit, (TQ*)direct, out_stride)
     if (nh != nkvh && sizeof(T) == 2) {
         if (staged) IC_DEC_LAUNCH((attn_decode_gqa_kernel<DH, true>), uint16_t);
         else IC_DEC_LAUNCH((attn_decode_gqa_kernel<DH, false>), uint16_t);
@@ -511,7 +522,7 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
     }
 #undef IC_DEC_LAUNCH
     int st = ic_launch_status();
-    if (st) return st;
+    if (st || nsplit == 1) return st;
     hipLaunchKernelGGL(attn_decode_reduce_kernel<T>, dim3(n_tok * nh), dim3(64), 0, stream, part_acc, part_ml,
                        tok_list, (T*)out, out_stride, nh, DH, nsplit);
     return ic_launch_status();

@@ -155,7 +155,7 @@ def test_rope_kv_write(dtype, nh, nkvh, dh, rot, page):
         _close(got[:, :nh][..., perm], adj, dtype)
 
 
-def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_width=0, groups=0):
+def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_width=0, groups=0, n_split=3):
     """lens: list of (past, new) per request.  Returns (got, want) [T, nh*dh].  table_width pads
     the block tables with unused columns; groups is passed to the prompt-portion kernel."""
     ops = _ops()
@@ -191,7 +191,6 @@ def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_w
         ops.attention_generic(q, out, kc, vc, btd, tr, ps, nh, nkvh, dh, page, scale, window or 0)
     elif impl == "decode":
         assert all(n == 1 for _, n in lens)
-        n_split = 3
         pa = torch.empty(T * nh * n_split * dh, device=DEV)
         pm = torch.empty(T * nh * n_split * 2, device=DEV)
         ops.attention_decode(q, out, kc, vc, btd, None, T, tr, ps, pa, pm, nh, nkvh, dh, page, scale,
@@ -222,9 +221,10 @@ def test_attention_generic(dtype, nh, nkvh, dh, page, window):
 @pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (5, 1, 64, 32), (8, 2, 128, 16),
                                               (16, 1, 128, 64)])
 @pytest.mark.parametrize("window", [None, 100])
-def test_attention_decode(dtype, nh, nkvh, dh, page, window):
+@pytest.mark.parametrize("n_split", [1, 3])          # one split writes the result itself, more go through the second pass
+def test_attention_decode(dtype, nh, nkvh, dh, page, window, n_split):
     lens = [(0, 1), (1, 1), (63, 1), (64, 1), (700, 1), (255, 1), (1031, 1)]
-    got, want = _attention_case(dtype, nh, nkvh, dh, page, lens, window, 12, "decode")
+    got, want = _attention_case(dtype, nh, nkvh, dh, page, lens, window, 12, "decode", n_split=n_split)
     _close(got, want, dtype, factor=3)
 
 
