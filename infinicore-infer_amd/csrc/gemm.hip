@@ -76,12 +76,18 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     __shared__ float ssum[WPB * 4][16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
-    // CSWIGLU: W = [gate rows (N/2); up rows (N/2)]; a block owns 16 gate rows and the matching
-    // 16 up rows and writes C[m][n] = up * silu(gate) for its 16 columns of the N/2 wide output.
+    // CSWIGLU: W = [gate rows (N/2); up rows (N/2)]; a block owns R = ceil((N/2) / blocks) <= 16 G
+    // gate rows (G = NT / 2 tiles of 16) and the matching up rows and writes C[m][n] = up * silu(gate)
+    // for its R columns of the N/2 wide output.  R need not be a multiple of 16: the launcher picks
+    // the number of blocks so that they fill the chip in one round where 16-row tiles would need
+    // a second, part-filled one.
     // CROPE: W = [q heads; k heads; v heads] (rows of dh).  A block owns 16 rows j.. of one q or k
     // head and the 16 rows j + dh/2.. that rotate with them, or 32 consecutive rows of a v head.
+    constexpr int G = CSWIGLU ? NT / 2 : 1;
     const int NO = CSWIGLU ? N / 2 : N;                      // output columns
-    int n0 = blockIdx.x * (CSWIGLU ? 16 : 16 * NT);
+    const int sw_cols = CSWIGLU ? (NO + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    int n0 = CSWIGLU ? blockIdx.x * sw_cols : blockIdx.x * (16 * NT);
+    const int sw_end = (n0 + sw_cols < NO) ? n0 + sw_cols : NO;   // CSWIGLU: one past the block's last column
     const int m0 = blockIdx.y * (16 * MT);
     int rope_head = 0, rope_j = 0;                           // CROPE: head and first index in the head
     bool rope_is_v = false;
@@ -101,9 +107,9 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     const uint16_t* wp[NT];
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
-        int base = CSWIGLU ? n0 + nt * NO : n0 + 16 * nt;
+        int base = CSWIGLU ? n0 + 16 * (nt % G) + (nt / G) * NO : n0 + 16 * nt;
         if (CROPE && nt == 1 && !rope_is_v) base = n0 + (rope.dh >> 1);
-        const int lim = CSWIGLU ? (nt + 1) * NO : N;
+        const int lim = CSWIGLU ? (nt / G) * NO + sw_end : N;
         const int nrow = (base + r < lim) ? base + r : lim - 1;
         wp[nt] = W + (size_t)nrow * ldw + 8 * kq;
     }
@@ -204,16 +210,18 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         for (int mt = 0; mt < MT; ++mt) {
             const int m = m0 + 16 * mt + r;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) {
-                float g = acc[0][mt][e], u = acc[NT - 1][mt][e];
+            for (int gi = 0; gi < G; ++gi)
 #pragma unroll
-                for (int w = 0; w < WPB - 1; ++w) { g += red[w][mt][lane][e]; u += red[w][(NT - 1) * MT + mt][lane][e]; }
-                // both projections are rounded to the output type first, as when they are stored
-                g = to_f32(from_f32<TC>(alpha * g));
-                u = to_f32(from_f32<TC>(alpha * u));
-                const int n = n0 + 4 * kq + e;
-                if (m < M && n < NO) C[(size_t)m * ldc + n] = from_f32<TC>(u * (g / (1.0f + expf(-g))));
-            }
+                for (int e = 0; e < 4; ++e) {
+                    float g = acc[gi][mt][e], u = acc[G + gi][mt][e];
+#pragma unroll
+                    for (int w = 0; w < WPB - 1; ++w) { g += red[w][gi * MT + mt][lane][e]; u += red[w][(G + gi) * MT + mt][lane][e]; }
+                    // both projections are rounded to the output type first, as when they are stored
+                    g = to_f32(from_f32<TC>(alpha * g));
+                    u = to_f32(from_f32<TC>(alpha * u));
+                    const int n = n0 + 16 * gi + 4 * kq + e;
+                    if (m < M && n < sw_end) C[(size_t)m * ldc + n] = from_f32<TC>(u * (g / (1.0f + expf(-g))));
+                }
         }
         return;
     }
@@ -308,16 +316,30 @@ static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int
 }
 
 // The gate/up projection with the activation in its epilogue: W [N, K] = [gate; up], C [M, N/2].
-template <typename TC, int WPB, int UN = 2>
+// G tiles of 16 gate rows (and as many of up rows) per block; `blocks` column blocks share the N/2 columns.
+template <typename TC, int WPB, int UN = 2, int G = 1>
 static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
-                               int ldc, bool aligned, const NormFuse& nf, hipStream_t stream) {
-    dim3 grid((N / 2 + 15) / 16, (M + 15) / 16), block(WPB * 64);
+                               int ldc, bool aligned, const NormFuse& nf, hipStream_t stream, int blocks = 0) {
+    if (blocks <= 0) blocks = (N / 2 + 16 * G - 1) / (16 * G);
+    dim3 grid(blocks, (M + 15) / 16), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, true, 1>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, true, 1>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2, 1, WPB, UN, false, 1>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, false, 1>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
+}
+
+// Compute units of the current device, asked once.
+static int compute_units() {
+    static int cus = 0;
+    if (cus == 0) {
+        int dev = 0, n = 0;
+        if (hipGetDevice(&dev) == hipSuccess &&
+            hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
+        else cus = 256;
+    }
+    return cus;
 }
 
 // NT weight tiles of 16 rows share one load of the A fragments; WPB waves split K.  Both are
@@ -366,6 +388,16 @@ IC_EXPORT int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype,
         if (M > 16 || (N & 1) || ldc < N / 2) return IC_ERR_ARG;
 #define IC_SW(WPB, UN) if (wpb == WPB && unroll == UN) { launch_gemm_swiglu<bf16, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, aligned, NormFuse{}, stream); return ic_launch_status(); }
         IC_SW(4, 2) IC_SW(4, 4) IC_SW(8, 2) IC_SW(8, 4) IC_SW(16, 2) IC_SW(16, 4)
+#undef IC_SW
+        return IC_ERR_UNSUPPORTED;
+    }
+    if (nt == -2) {                                 // the SwiGLU variant with two tiles per block, one block per compute unit
+        if (M > 16 || (N & 1) || ldc < N / 2) return IC_ERR_ARG;
+        const int cols = (N / 2 + compute_units() - 1) / compute_units();
+        if (cols > 32) return IC_ERR_UNSUPPORTED;
+        const int blocks = (N / 2 + cols - 1) / cols;
+#define IC_SW(WPB, UN) if (wpb == WPB && unroll == UN) { launch_gemm_swiglu<bf16, WPB, UN, 2>(A, W, C, M, N, K, lda, ldw, ldc, aligned, NormFuse{}, stream, blocks); return ic_launch_status(); }
+        IC_SW(4, 2) IC_SW(4, 4) IC_SW(8, 2) IC_SW(8, 4) IC_SW(16, 2)
 #undef IC_SW
         return IC_ERR_UNSUPPORTED;
     }
@@ -427,12 +459,19 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
         return ic_launch_status();
     }
     if (c_mode == 1) {
-        const int tiles = (N / 2 + 15) / 16;
+        const int tiles = (N / 2 + 15) / 16, cus = compute_units();
+        // Between one and two 16-column tiles per compute unit the second round of blocks would be part-filled:
+        // then every block takes ceil(columns / units) columns (two tiles, the second one partial) and one round does it.
+        const int cols = (N / 2 + cus - 1) / cus;
+        const bool one_round = tiles > cus && cols <= 32;
+        const int blocks = one_round ? (N / 2 + cols - 1) / cols : 0;
         if (c_dtype == IC_F32) {
-            if (tiles < 300) launch_gemm_swiglu<float, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
+            if (one_round) launch_gemm_swiglu<float, 8, 2, 2>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream, blocks);
+            else if (tiles < 300) launch_gemm_swiglu<float, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
             else launch_gemm_swiglu<float, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
         } else {
-            if (tiles < 300) launch_gemm_swiglu<bf16, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
+            if (one_round) launch_gemm_swiglu<bf16, 8, 2, 2>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream, blocks);
+            else if (tiles < 300) launch_gemm_swiglu<bf16, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
             else launch_gemm_swiglu<bf16, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
         }
         return ic_launch_status();
