@@ -88,6 +88,10 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     const int sw_cols = CSWIGLU ? (NO + (int)gridDim.x - 1) / (int)gridDim.x : 0;
     int n0 = CSWIGLU ? blockIdx.x * sw_cols : blockIdx.x * (16 * NT);
     const int sw_end = (n0 + sw_cols < NO) ? n0 + sw_cols : NO;   // CSWIGLU: one past the block's last column
+    // CRESID: a block owns ceil(N / blocks) <= 16 columns, so that few columns still make a block per compute unit
+    const int rs_cols = CRESID ? (N + (int)gridDim.x - 1) / (int)gridDim.x : 0;
+    if (CRESID) n0 = blockIdx.x * rs_cols;
+    const int rs_end = (n0 + rs_cols < N) ? n0 + rs_cols : N;
     const int m0 = blockIdx.y * (16 * MT);
     int rope_head = 0, rope_j = 0;                           // CROPE: head and first index in the head
     bool rope_is_v = false;
@@ -109,7 +113,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     for (int nt = 0; nt < NT; ++nt) {
         int base = CSWIGLU ? n0 + 16 * (nt % G) + (nt / G) * NO : n0 + 16 * nt;
         if (CROPE && nt == 1 && !rope_is_v) base = n0 + (rope.dh >> 1);
-        const int lim = CSWIGLU ? (nt / G) * NO + sw_end : N;
+        const int lim = CSWIGLU ? (nt / G) * NO + sw_end : (CRESID ? rs_end : N);
         const int nrow = (base + r < lim) ? base + r : lim - 1;
         wp[nt] = W + (size_t)nrow * ldw + 8 * kq;
     }
@@ -141,7 +145,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
         for (int e = 0; e < 4; ++e) {
             const int n = n0 + 4 * kq + e;
-            if (n < N) { xres[e] = nf.x[(size_t)(m0 + r) * nf.ldx + n]; gres[e] = nf.g[n]; }
+            if (n < rs_end) { xres[e] = nf.x[(size_t)(m0 + r) * nf.ldx + n]; gres[e] = nf.g[n]; }
         }
     }
 
@@ -274,7 +278,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
             for (int w = 0; w < WPB - 1; ++w) v += red[w][0][lane][e];
             const int n = n0 + 4 * kq + e;
-            if (m < M && n < N) {
+            if (m < M && n < rs_end) {
                 const float d = to_f32(from_f32<TC>(alpha * v));     // the branch's output as it would be stored
                 const float h = xres[e] + nf.rscale * d;
                 nf.x[(size_t)m * nf.ldx + n] = h;
@@ -305,8 +309,8 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 
 template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0>
 static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
-                        int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream) {
-    dim3 grid((N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
+                        int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream, int blocks = 0) {
+    dim3 grid(blocks > 0 ? blocks : (N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
     if (aligned)
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
@@ -433,7 +437,14 @@ static bool norm_fuse_args(const IcRowFactor* rf, const IcResidualNorm* tail, in
 }
 
 // Column blocks (= sums of squares per row) that c_mode 2 writes for an N wide product.
-IC_EXPORT int ic_gemm_nt_residual_parts(int N) { return (N + 15) / 16; }
+// (one block per compute unit when 16-column tiles would be fewer than the units)
+static int compute_units();
+IC_EXPORT int ic_gemm_nt_residual_parts(int N) {
+    const int tiles = (N + 15) / 16, cus = compute_units();
+    if (tiles >= cus || N <= 0) return tiles;
+    const int cols = (N + cus - 1) / cus;
+    return (N + cols - 1) / cols;
+}
 
 // c_mode 0: C [M, N] = alpha * A W^T.  c_mode 1 (M <= 16, N even, alpha ignored): W = [gate; up] and
 // C [M, N/2] = up * silu(gate), both projections rounded to C's type before the activation.
@@ -454,8 +465,9 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
     if (c_mode == 2) {
         // a long K over few columns (the down projection) does better with fewer, longer waves (from a sweep)
-        if (K > 2 * N) launch_gemm<bf16, 1, 1, 8, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream);
-        else launch_gemm<bf16, 1, 1, 16, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream);
+        const int blocks = ic_gemm_nt_residual_parts(N);
+        if (K > 2 * N) launch_gemm<bf16, 1, 1, 8, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
+        else launch_gemm<bf16, 1, 1, 16, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
         return ic_launch_status();
     }
     if (c_mode == 1) {

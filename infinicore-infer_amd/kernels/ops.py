@@ -275,7 +275,7 @@ MAX_SUMSQ_PARTS = 256      # column blocks of sums of squares a product can take
 
 def residual_parts(n: int) -> int:
     """Column blocks of sums of squares that gemm_nt(..., residual=...) writes for an n wide product."""
-    return (n + 15) // 16
+    return int(get_lib().ic_gemm_nt_residual_parts(int(n)))
 
 
 def _row_factor(row_factor, M, what):
