@@ -82,8 +82,9 @@ int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int ld
 // descriptors at the first call of a shape; workspace is device memory passed in by the caller.
 int ic_matmul_supported(int a_dtype, int c_dtype);
 int ic_matmul(const void* A, int a_dtype, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, void* workspace, long long workspace_bytes, hipStream_t stream);
-// Times the algorithms the library proposes for this shape and keeps the fastest; returns how many were tried.
-int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, void* workspace, long long workspace_bytes, int reps, hipStream_t stream);
+// Times the algorithms the library has for this shape and keeps the fastest; returns how many were tried.
+// flush (or nullptr): memory larger than the caches, overwritten before every timed launch so that operands come from memory.
+int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, void* workspace, long long workspace_bytes, void* flush, long long flush_bytes, int reps, hipStream_t stream);
 
 // ---- sampling.hip -----------------------------------------------------------------------------------
 // Greedy choice per row; scratch_val / scratch_idx: 64 * n_rows elements.

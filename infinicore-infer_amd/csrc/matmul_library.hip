@@ -126,10 +126,14 @@ IC_EXPORT int ic_matmul(const void* A, int a_dtype, const void* W, void* C, int 
 // Times every algorithm the library proposes for this product (reps launches each, after one to warm up) on
 // `stream` and keeps the fastest, if it beats the library's first choice by 3 %, for later ic_matmul calls of the
 // same shape.  Synchronises the stream.
+// flush (may be nullptr): device memory, larger than the chip's caches, that is overwritten before every timed
+// launch, so that the operands come from memory as a model's weights do and not from the last launch's cache lines.
 // Returns the number of algorithms tried (>= 1) or an error code (< 0).
 IC_EXPORT int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C, int c_dtype, int M, int N, int K, int lda,
-                             int ldw, int ldc, void* workspace, long long workspace_bytes, int reps, hipStream_t stream) {
-    if (!args_ok(A, a_dtype, W, C, c_dtype, M, N, K, lda, ldw, ldc) || workspace_bytes < 0 || reps < 1) return IC_ERR_ARG;
+                             int ldw, int ldc, void* workspace, long long workspace_bytes, void* flush, long long flush_bytes,
+                             int reps, hipStream_t stream) {
+    if (!args_ok(A, a_dtype, W, C, c_dtype, M, N, K, lda, ldw, ldc) || workspace_bytes < 0 || reps < 1 || flush_bytes < 0) return IC_ERR_ARG;
+    if (!flush) flush_bytes = 0;
     std::lock_guard<std::mutex> lock(g_mu);
     Plan* p = nullptr;
     const int st = plan_for(Key{a_dtype, c_dtype, M, N, K, lda, ldw, ldc}, (size_t)workspace_bytes, &p);
@@ -158,13 +162,17 @@ IC_EXPORT int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C,
     if (hipEventCreate(&e1) != hipSuccess) { hipEventDestroy(e0); return IC_ERR_LIBRARY; }
     auto time_one = [&](int i, int n) -> float {            // ms per launch, < 0: failed
         if (run(*p, i, A, W, C, 1.0f, workspace, (size_t)workspace_bytes, stream) != IC_OK) return -1.f;
-        hipEventRecord(e0, stream);
-        bool ok = true;
-        for (int r = 0; r < n && ok; ++r) ok = run(*p, i, A, W, C, 1.0f, workspace, (size_t)workspace_bytes, stream) == IC_OK;
-        hipEventRecord(e1, stream);
-        float ms = 0.f;
-        if (hipEventSynchronize(e1) != hipSuccess || !ok || hipEventElapsedTime(&ms, e0, e1) != hipSuccess) return -1.f;
-        return ms / n;
+        float total = 0.f;
+        for (int r = 0; r < n; ++r) {
+            if (flush_bytes > 0 && hipMemsetAsync(flush, r & 1, (size_t)flush_bytes, stream) != hipSuccess) return -1.f;
+            hipEventRecord(e0, stream);
+            const bool ok = run(*p, i, A, W, C, 1.0f, workspace, (size_t)workspace_bytes, stream) == IC_OK;
+            hipEventRecord(e1, stream);
+            float ms = 0.f;
+            if (hipEventSynchronize(e1) != hipSuccess || !ok || hipEventElapsedTime(&ms, e0, e1) != hipSuccess) return -1.f;
+            total += ms;
+        }
+        return total / n;
     };
     // first round: one timed launch each; second round: the eight best and the first choice, reps launches each
     std::vector<std::pair<float, int>> quick;

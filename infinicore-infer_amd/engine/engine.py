@@ -332,11 +332,14 @@ class Engine:
     def tune_library_products(self, token_counts: Sequence[int]) -> None:
         """Let the library's matrix products for prompt portions of the given token counts use their
         fastest algorithm: one dummy step per count is run in which every library product first times
-        the algorithms the library proposes for its shape on the device and keeps the best.  Other
+        the algorithms the library has for its shape on the device and keeps the best.  Between
+        timed launches 512 MB of scratch memory are overwritten: in a model every product's weights
+        come from memory, not from the cache lines a repeated launch would find.  Other
         shapes keep the library's first choice and cost nothing.  Optional; results live for this
         process."""
         from ..parts import linear as _linear
         _linear.TUNE_LIBRARY = True
+        _linear.TUNE_FLUSH = torch.empty(512 << 20, dtype=torch.uint8, device=self.device)
         try:
             for n in token_counts:
                 rid = ("tune", n)
@@ -345,6 +348,7 @@ class Engine:
             torch.cuda.synchronize()
         finally:
             _linear.TUNE_LIBRARY = False
+            _linear.TUNE_FLUSH = None
 
     # ---- sampling --------------------------------------------------------------------------------------
     def sample(self, logits, temperature=None, top_k=None, top_p=None, uniform=None) -> List[int]:

@@ -370,13 +370,19 @@ def matmul_library(a, w, out, alpha: float = 1.0):
     return out
 
 
-def matmul_library_tune(a, w, out, reps: int = 5) -> int:
-    """Times the library's algorithms for this product's shape and keeps the fastest; returns how many it tried."""
+def matmul_library_tune(a, w, out, reps: int = 5, flush=None) -> int:
+    """Times the library's algorithms for this product's shape and keeps the fastest; returns how many it tried.
+    flush: a device tensor larger than the chip's caches; it is overwritten before every timed launch, so that the
+    algorithms are compared with operands that come from memory, as a model's weights do."""
     M, N, K = _matmul_args(a, w, out, "matmul_library_tune")
     ws = _workspace(a.device)
+    if flush is not None:
+        _dev(a, flush)
+        _need(flush.is_contiguous(), "matmul_library_tune: flush must be contiguous")
     n = get_lib().ic_matmul_tune(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), out.data_ptr(), dtype_code(out.dtype),
-                                 M, N, K, a.stride(0), w.stride(0), out.stride(0), ws.data_ptr(), ws.numel(), int(reps),
-                                 _stream())
+                                 M, N, K, a.stride(0), w.stride(0), out.stride(0), ws.data_ptr(), ws.numel(),
+                                 flush.data_ptr() if flush is not None else None,
+                                 flush.numel() * flush.element_size() if flush is not None else 0, int(reps), _stream())
     if n < 0:
         raise KernelError("matmul_library_tune failed with %d for %d x %d x %d" % (n, M, N, K))
     return n

@@ -17,6 +17,7 @@ torch.backends.cudnn.allow_tf32 = False
 
 FEW_ROWS = 16          # up to here the package's own kernel beats the library on MI355X
 TUNE_LIBRARY = False   # while True, every library product times the library's algorithms for its shape first
+TUNE_FLUSH = None      # while tuning: a tensor larger than the caches, overwritten before every timed launch
 _tuned = set()
 
 
@@ -29,7 +30,7 @@ def _library(x, w, out, alpha: float = 1.0):
         if key not in _tuned:
             _tuned.add(key)
             try:
-                ops.matmul_library_tune(x, w, out)
+                ops.matmul_library_tune(x, w, out, flush=TUNE_FLUSH)
             except ops.KernelError:
                 pass
     try:

@@ -345,6 +345,28 @@ def test_gemm_nt(cdtype, M, N, K):
     _close(out, want, cdtype, factor=2)
 
 
+@pytest.mark.parametrize("dtype,cdtype", [(torch.bfloat16, torch.bfloat16), (torch.bfloat16, torch.float32),
+                                          (torch.float32, torch.float32)])
+@pytest.mark.parametrize("M,N,K", [(40, 331, 200), (300, 1000, 344)])
+def test_library_product_before_and_after_timing_its_algorithms(dtype, cdtype, M, N, K):
+    """The library product called directly: with the library's first choice, and again after every
+    algorithm was timed (with a buffer overwritten between the launches) and the fastest kept."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(21)
+    a = torch.randn(M, K, generator=g).to(dtype)
+    w = torch.randn(N, K, generator=g).to(dtype)
+    want = 0.25 * P.plain_linear(a, w)
+    ad, wd = a.to(DEV), w.to(DEV)
+    out = torch.full((M, N), float("nan"), dtype=cdtype, device=DEV)
+    ops.matmul_library(ad, wd, out, 0.25)
+    _close(out, want, cdtype if dtype == torch.bfloat16 else torch.float32, factor=2)
+    flush = torch.empty(8 << 20, dtype=torch.uint8, device=DEV)
+    assert ops.matmul_library_tune(ad, wd, out, reps=2, flush=flush) >= 1
+    out.fill_(float("nan"))
+    ops.matmul_library(ad, wd, out, 0.25)
+    _close(out, want, cdtype if dtype == torch.bfloat16 else torch.float32, factor=2)
+
+
 def test_library_float32_product_is_true_float32():
     """The float32 path's matrix products must not run in a reduced-precision mode."""
     from infinicore_infer_amd.parts.linear import linear
