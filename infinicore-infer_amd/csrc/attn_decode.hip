@@ -248,16 +248,19 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
     }
 }
 
-// Grid (tokens * heads), one wave.  Lane s holds split s (at most 64 splits): the
-// weights exp(m_s - max) come from one wave reduction; every lane then sums its
-// output dims over the splits with independent loads.
+// Grid (tokens * heads), four waves.  Lane s of every wave holds split s (at most 64 splits): the
+// weights exp(m_s - max) come from one wave reduction.  Thread (d, g) then sums output dim d over
+// the splits g, g + G, .. (G = 256 / dh groups) with independent loads, and the groups meet in LDS:
+// with many splits (few kv heads, few requests) one wave alone would walk them one after the other.
+constexpr int kRedThreads = 256;
 template <typename T>
-__global__ void __launch_bounds__(64)
+__global__ void __launch_bounds__(kRedThreads)
 attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                           const int* __restrict__ tok_list, T* __restrict__ out,
                           int out_stride, int nh, int dh, int nsplit) {
     __shared__ float wgt[64];
-    const int n = blockIdx.x / nh, h = blockIdx.x % nh, lane = threadIdx.x;
+    __shared__ float grp[kRedThreads];
+    const int n = blockIdx.x / nh, h = blockIdx.x % nh, tid = threadIdx.x, lane = tid & 63;
     const int t = tok_list ? tok_list[n] : n;
     const size_t base = ((size_t)n * nh + h) * nsplit;
     float ms = -INFINITY, ls = 0.f;
@@ -265,13 +268,20 @@ attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __res
     const float mm = wave_max(ms);
     const float w = (ms == -INFINITY) ? 0.f : expf(ms - mm);
     const float inv = 1.0f / wave_sum(ls * w);
-    wgt[lane] = w;
+    if (tid < 64) wgt[lane] = w;
     __syncthreads();
-    for (int d = lane; d < dh; d += 64) {
-        float a = 0.f;
-#pragma unroll 4
-        for (int s = 0; s < nsplit; ++s) a += part_acc[(base + s) * dh + d] * wgt[s];
-        out[(size_t)t * out_stride + (size_t)h * dh + d] = from_f32<T>(a * inv);
+    // dh <= 256: G >= 1 groups of dh threads
+    const int G = kRedThreads / dh, g = tid / dh, d = tid - g * dh;
+    float a = 0.f;
+    if (g < G) {
+#pragma unroll 8
+        for (int s = g; s < nsplit; s += G) a += part_acc[(base + s) * dh + d] * wgt[s];
+    }
+    grp[tid] = a;
+    __syncthreads();
+    if (tid < dh) {
+        for (int j = 1; j < G; ++j) a += grp[j * dh + tid];
+        out[(size_t)t * out_stride + (size_t)h * dh + tid] = from_f32<T>(a * inv);
     }
 }
 
@@ -523,7 +533,7 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
 #undef IC_DEC_LAUNCH
     int st = ic_launch_status();
     if (st || nsplit == 1) return st;
-    hipLaunchKernelGGL(attn_decode_reduce_kernel<T>, dim3(n_tok * nh), dim3(64), 0, stream, part_acc, part_ml,
+    hipLaunchKernelGGL(attn_decode_reduce_kernel<T>, dim3(n_tok * nh), dim3(kRedThreads), 0, stream, part_acc, part_ml,
                        tok_list, (T*)out, out_stride, nh, DH, nsplit);
     return ic_launch_status();
 }

@@ -85,14 +85,21 @@ class StepContext:
             v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache)
         return v
 
-    def decode_splits(self, n_kv_heads: int, window: int = 0) -> int:
+    def decode_splits(self, n_kv_heads: int, window: int = 0, matrix_core_tiles_of: int = 0) -> int:
         """How many ways to split the keys of single-token rows.  From sweeps on MI355X with a
-        cold cache: few (row, kv head) pairs want about 1.75 blocks per compute unit however short
-        the loops get; more pairs want about 3.4 per unit; a split never gets fewer than 64 keys."""
+        cold cache.  One query head per kv head (a wave walks keys with vector instructions): few
+        (row, kv head) pairs want about 1.75 blocks per compute unit however short the loops get;
+        more pairs want about 3.4 per unit.  Grouped query heads on the matrix cores
+        (``matrix_core_tiles_of`` = the head size): a wave has a whole 32-key tile in flight, so
+        128 / head size blocks per unit are enough and more only add partial results to merge.
+        A split never gets fewer than 64 keys."""
         if self.fixed_decode_splits is not None:
             return self.fixed_decode_splits
         keys = self.max_context if not window else min(self.max_context, window)
         base = max(1, self.n_decode_rows * n_kv_heads)
-        per_unit = 1.75 if base < 0.6 * self.cu_count else 3.4
+        if matrix_core_tiles_of:
+            per_unit = 128.0 / matrix_core_tiles_of
+        else:
+            per_unit = 1.75 if base < 0.6 * self.cu_count else 3.4
         want = max(1, int(per_unit * self.cu_count / base + 0.5))
         return int(max(1, min(want, max(1, keys // 64), 64)))

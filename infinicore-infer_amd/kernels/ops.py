@@ -183,6 +183,12 @@ def attention_decode_supported(dtype, head_dim: int) -> bool:
     return bool(get_lib().ic_attn_decode_supported(dtype_code(dtype), head_dim))
 
 
+def attention_decode_on_matrix_cores(dtype, n_heads: int, n_kv_heads: int) -> bool:
+    """True when attention_decode runs its grouped-query kernel (bfloat16, several query heads per
+    kv head): that kernel wants fewer key splits than the one-head-per-wave kernel."""
+    return dtype == torch.bfloat16 and n_heads != n_kv_heads
+
+
 def attention_decode(q, out, kcache, vcache, block_tables, tok_list, n_tok, token_req, positions, part_acc,
                      part_ml, n_heads, n_kv_heads, head_dim, page_size, scale: float, window: int, n_split: int):
     """Split-key attention of the single tokens listed in tok_list (None: rows 0..n_tok-1)."""
