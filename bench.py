@@ -124,6 +124,64 @@ def time_decode(engine, batch, steps, warmup, vocab, seed=0):
     return dt / steps, (ctx0 + ctx1) / 2.0
 
 
+def run_mixed(args):
+    """The 1B-shaped configuration's workload: 64 requests with prompts of 128..2,048 tokens go through the
+    scheduler, which cuts the prompts into portions of 512 under a token budget per step and decodes the
+    running requests beside them.  One JSON line: all tokens (prompt and generated) per second."""
+    import random
+    from infinicore_infer_amd.engine.scheduler import Scheduler
+    from infinicore_infer_amd.engine.tasks import InferTask
+    n_req, gen, chunk, budget = args.requests, args.steps, 512, args.token_budget
+    rnd = random.Random(0)
+    lens = [rnd.randint(128, 2048) for _ in range(n_req)]
+    pool = sum((l + gen + args.page_size - 1) // args.page_size * args.page_size for l in lens) + 64 * args.page_size
+    engine, conf = build_engine(args.layers, pool, n_req, args.page_size)
+    if not args.no_tune:
+        engine.tune_library_products([b for b in (n_req,) if b > 16])
+    g = torch.Generator().manual_seed(1)
+    prompts = [torch.randint(0, conf.vocab_size, (l,), generator=g).tolist() for l in lens]
+
+    def run():
+        sch = Scheduler(engine, max_batch_tokens=budget, chunk_size=chunk)
+        for i, toks in enumerate(prompts):
+            sch.add(InferTask(i, toks, conf.max_position_embeddings, temperature=0.0, topk=1, end_tokens=[], max_new_tokens=gen))
+        _sync()
+        t0 = time.perf_counter()
+        steps = []
+        while sch.has_unfinished():
+            s0 = time.perf_counter()
+            sch.step()
+            steps.append((time.perf_counter() - s0, sum(n for _, _, n in sch.last_plan)))
+        _sync()
+        return time.perf_counter() - t0, steps, sch.n_preempted
+
+    run()                                            # one untimed pass: buffers grow, graphs are recorded
+    dt, steps, preempted = run()
+    total = sum(lens) + n_req * gen
+    mixed = [s for s in steps if s[1] > n_req]
+    dec = [s for s in steps if s[1] <= n_req]
+    out = {
+        "metric": "tokens/s (prompt + generated) through the scheduler, %d requests, prompts 128..2048, portions of %d "
+                  "(MiniCPM-%s-shaped)" % (n_req, chunk, args.shape.upper()),
+        "value": round(total / dt, 1), "unit": "tokens/s", "n_gpus": 1, "steps": len(steps), "warmup": 1,
+        "ms_per_step": round(dt / len(steps) * 1e3, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
+        "dtype": "bf16", "data": "synthetic (seeded random weights N(0,0.1) and token ids)",
+        "config": {
+            "model": "MiniCPM-%s-shaped" % args.shape.upper(), "layers": conf.num_hidden_layers, "layers_of_config": MODEL["num_hidden_layers"],
+            "hidden": conf.hidden_size, "heads": conf.num_attention_heads, "kv_heads": conf.num_key_value_heads,
+            "head_dim": conf.head_dim, "intermediate": conf.intermediate_size, "vocab": conf.vocab_size,
+            "requests": n_req, "prompt_tokens": sum(lens), "generated_each": gen, "token_budget": budget, "portion": chunk,
+            "page_size": args.page_size, "parallelism": "single-gpu", "sampling": "greedy on device",
+        },
+        "mixed_steps": {"count": len(mixed), "mean_ms": round(1e3 * sum(s[0] for s in mixed) / max(1, len(mixed)), 3),
+                        "mean_tokens": round(sum(s[1] for s in mixed) / max(1, len(mixed)), 1)},
+        "decode_steps": {"count": len(dec), "mean_ms": round(1e3 * sum(s[0] for s in dec) / max(1, len(dec)), 3)},
+        "preempted": preempted,
+    }
+    print(json.dumps(out))
+    return 0
+
+
 def main():
     global BATCH, MODEL, PROMPT
     ap = argparse.ArgumentParser()
@@ -131,7 +189,12 @@ def main():
     ap.add_argument("--steps", type=int, default=128)
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
-    ap.add_argument("--shape", default="2b", choices=sorted(SHAPES), help="2b is the benchmark's configuration")
+    ap.add_argument("--shape", default=None, choices=sorted(SHAPES), help="2b is the benchmark's configuration (default; 1b for --workload mixed)")
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
+                    help="decode: the benchmark (prefill of one prompt, decode steps at fixed batches); "
+                         "mixed: 64 requests of 128..2048 prompt tokens through the scheduler, --steps tokens generated each")
+    ap.add_argument("--requests", type=int, default=64, help="--workload mixed: number of requests")
+    ap.add_argument("--token-budget", type=int, default=1024, help="--workload mixed: tokens per step")
     ap.add_argument("--prompt", type=int, default=PROMPT)
     ap.add_argument("--page-size", type=int, default=64)
     ap.add_argument("--no-points", action="store_true", help="skip the batch 1 and 64 points")
@@ -144,7 +207,13 @@ def main():
         return 2
 
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    if args.shape is None:
+        args.shape = "1b" if args.workload == "mixed" else "2b"
     MODEL, PROMPT = SHAPES[args.shape], args.prompt
+    if args.workload == "mixed":
+        if args.steps == ap.get_default("steps"):
+            args.steps = 64
+        return run_mixed(args)
     per_req = PROMPT + args.warmup + args.steps + 64
     per_req = (per_req + 63) // 64 * 64
     BATCH = args.batch
