@@ -113,6 +113,32 @@ def test_first_tokens(tmp_path_factory, name, dname, dtype, tol):
     H.compare(H.run_trace(engine, whole), ref, tol, "first tokens as one portion")
 
 
+@pytest.mark.parametrize("dname,dtype,tol", DTYPES)
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_decoding_twenty_requests_at_once(tmp_path_factory, name, dname, dtype, tol):
+    """More rows than the few-row kernels take (16): the prompts of twenty requests in one step, then
+    every request's next token in one step, eight times over (library products, the unfused
+    norm, rotary and activation kernels, a recorded graph of that batch size)."""
+    from infinicore_infer_amd.engine import Engine
+    cfg = H.CONFIGS[name][0]
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), name)
+    n_req, n_dec = 20, 8
+    lens = [3 + (7 * i) % 41 for i in range(n_req)]
+    requests = {"m%d" % i: H.random_tokens(cfg["vocab_size"], lens[i] + n_dec, 500 + i) for i in range(n_req)}
+    steps = [{"step": 0, "end": [],
+              "entries": [{"id": k, "tokens": t[:lens[i]], "want": [lens[i] - 1]} for i, (k, t) in enumerate(requests.items())]}]
+    for j in range(n_dec):
+        steps.append({"step": j + 1, "end": list(requests) if j == n_dec - 1 else [],
+                      "entries": [{"id": k, "tokens": [t[lens[i] + j]], "want": [0]} for i, (k, t) in enumerate(requests.items())]})
+    engine = Engine.from_dir(folder, dtype=dtype, max_tokens=n_req * 64, page_size=16, max_requests=n_req)
+    got = H.run_trace(engine, steps)
+    ref = H.plain_logits(cfg, H.load_state_dict(folder), requests, dtype == torch.bfloat16)
+    assert len(got) == n_req * (1 + n_dec)
+    H.compare(got, ref, tol, "%s %s twenty requests" % (name, dname))
+    assert engine.graph_replays == n_dec
+    engine.cache.check_invariants()
+
+
 def test_out_of_pages_changes_nothing(tmp_path_factory):
     from infinicore_infer_amd.cache import OutOfPages
     from infinicore_infer_amd.engine import StepEntry
