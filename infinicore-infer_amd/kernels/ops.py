@@ -340,9 +340,12 @@ MATMUL_WORKSPACE_BYTES = 64 << 20
 
 
 def _workspace(device):
-    ws = _matmul_workspace.get(device)
+    """The library's scratch memory: one buffer per device and stream, since products that run at the
+    same time on different streams must not share it (some algorithms keep flags and partial sums there)."""
+    key = (device, _stream())
+    ws = _matmul_workspace.get(key)
     if ws is None:
-        ws = _matmul_workspace[device] = torch.empty(MATMUL_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
+        ws = _matmul_workspace[key] = torch.empty(MATMUL_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
     return ws
 
 
