@@ -18,18 +18,25 @@ class Workspace:
 
     def __init__(self, device):
         self.device = device
-        self._bufs: Dict[str, torch.Tensor] = {}
+        self._bufs: Dict[tuple, torch.Tensor] = {}
+        self._views: Dict[tuple, tuple] = {}     # (name, dtype) -> (shape, view): the view handed out last
 
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:
+        key = (name, dtype)
+        shape = tuple(shape)
+        last = self._views.get(key)
+        if last is not None and last[0] == shape:       # the usual case: the same shape as last time
+            return last[1]
         n = 1
         for s in shape:
             n *= int(s)
-        key = "%s/%s" % (name, str(dtype))
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < n:
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = buf
-        return buf[:n].view(*shape)
+        view = buf[:n].view(*shape)
+        self._views[key] = (shape, view)
+        return view
 
     def bytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())
