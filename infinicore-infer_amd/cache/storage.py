@@ -28,6 +28,7 @@ class CacheStorage:
             for i, s in enumerate(spec.slots):
                 self._slot_index[s] = (g, i)
         self.state: Dict[int, torch.Tensor] = {}               # cache slot -> [max_requests, ...]
+        self._kv_views: Dict[int, tuple] = {}
 
     def add_state(self, slot: int, max_requests: int, shape, dtype) -> torch.Tensor:
         t = torch.zeros((max_requests,) + tuple(shape), dtype=dtype, device=self.device)
@@ -38,9 +39,12 @@ class CacheStorage:
         return self._slot_index[slot][0]
 
     def kv(self, slot: int):
-        """(K plane, V plane) of a cache slot."""
-        g, i = self._slot_index[slot]
-        return self.group_planes[g][i, 0], self.group_planes[g][i, 1]
+        """(K plane, V plane) of a cache slot (views made once: the planes never move)."""
+        kv = self._kv_views.get(slot)
+        if kv is None:
+            g, i = self._slot_index[slot]
+            kv = self._kv_views[slot] = (self.group_planes[g][i, 0], self.group_planes[g][i, 1])
+        return kv
 
     def zero_state(self, state_slot: int) -> None:
         for t in self.state.values():

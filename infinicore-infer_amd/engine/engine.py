@@ -291,12 +291,12 @@ class Engine:
         ctx.max_position = max(p0 + n - 1 for p0, n in zip(starts, lens))
         ctx.max_context = _context_bucket(max_ctx) if max_ctx else 0
         ctx.cu_count = self.cu_count
+        group_views = [(view("slots%d" % g), view("tables%d" % g).view(R, group_maxb[g])) for g in range(n_groups)]
         for slot in range(self.model.spec.num_cache_slots()):
             if slot in self._slot_group:
-                g = self._slot_group[slot]
+                slots, tables_g = group_views[self._slot_group[slot]]
                 k, v = self.storage.kv(slot)
-                ctx._views[slot] = LayerCacheView(k=k, v=v, slots=view("slots%d" % g),
-                                                  block_tables=view("tables%d" % g).view(R, group_maxb[g]))
+                ctx._views[slot] = LayerCacheView(k=k, v=v, slots=slots, block_tables=tables_g)
             else:
                 ctx._views[slot] = LayerCacheView(state=self.storage.state.get(slot))
         return ctx

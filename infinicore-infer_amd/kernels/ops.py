@@ -4,7 +4,7 @@ then launches on torch's current stream.  Nothing here computes on the CPU.
 """
 import torch
 
-from .lib import KernelError, check, get_lib
+from .lib import IcResidualNorm, IcRowFactor, KernelError, check, get_lib
 
 F32, BF16 = 0, 1
 _DT = {torch.float32: F32, torch.bfloat16: BF16}
@@ -288,7 +288,6 @@ def _row_factor(row_factor, M, what):
     """row_factor = (sumsq float32 [n_parts, 16], width, eps) -> the C struct (or None)."""
     if row_factor is None:
         return None
-    from .lib import IcRowFactor
     sumsq, width, eps = row_factor
     _dev(sumsq)
     _need(M <= 16, what + ": row factors need at most 16 rows")
@@ -317,7 +316,6 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
     rn = None
     mode = 1 if swiglu_output else 0
     if residual is not None:
-        from .lib import IcResidualNorm
         x, weight, beta, sumsq_out = residual
         _dev(x, weight, sumsq_out)
         _need(not swiglu_output and M <= 16 and out.dtype == torch.bfloat16, "gemm_nt: residual epilogue needs M <= 16 and bfloat16 out")

@@ -12,7 +12,7 @@ import torch
 
 from ..kernels import ops
 from ..weights.loader import WeightSpec
-from .base import Part, register_part
+from .base import DeferredRows, Part, register_part
 from .linear import linear
 
 
@@ -63,7 +63,6 @@ class LMHead(Part):
 
     def forward(self, x, rows, final_norm, ctx):
         """Float32 logits [len(rows), vocab] of the residual rows ``rows``."""
-        from .base import DeferredRows
         if isinstance(x, DeferredRows):
             # every row in order, the final norm half done: its row factors go into the product
             logits = ctx.ws.buffer("logits", (x.shape[0], self.vocab_size), torch.float32)

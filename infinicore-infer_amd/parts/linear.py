@@ -10,6 +10,7 @@ switched off.
 import torch
 
 from ..kernels import ops
+from .base import DeferredRows
 
 # float32 products must be true float32.
 torch.backends.cuda.matmul.allow_tf32 = False
@@ -51,7 +52,6 @@ def own_kernel_applies(M, x_dtype, w_dtype, out_dtype, impl: str) -> bool:
 def linear(x, w, out, impl: str = "auto", alpha: float = 1.0):
     """out[M, N] = alpha * x[M, K] @ w[N, K]^T.  out may be float32 when x is bfloat16.  x may be
     ``DeferredRows``: the row factors are applied to the result by the own kernel, or to x first."""
-    from .base import DeferredRows
     if isinstance(x, DeferredRows):
         if own_kernel_applies(x.shape[0], x.dtype, w.dtype, out.dtype, impl):
             return ops.gemm_nt(x.values, w, out, alpha=alpha, row_factor=x.row_factor())
@@ -71,7 +71,6 @@ def linear_tail(x, w, tail, ws, name: str, impl: str = "auto"):
     """The last projection of a part with the residual add and the following norm's weight in its
     epilogue: returns ``DeferredRows`` for that norm, or None when this step cannot be done so
     (many rows, float32, a width beyond the kernel's) and the caller computes the plain product."""
-    from .base import DeferredRows
     M, N = x.shape[0], w.shape[0]
     if tail is None or not own_kernel_applies(M, x.dtype, w.dtype, torch.bfloat16, impl):
         return None

@@ -17,7 +17,8 @@ import math
 import torch
 
 from ..kernels import ops
-from .base import PositionEncoding, register_part
+from .base import DeferredRows, PositionEncoding, register_part
+from .linear import FEW_ROWS
 
 
 def rotary_tables(head_dim, theta, max_positions, scaling=None, rot_dim=None):
@@ -71,8 +72,6 @@ class Rotary(PositionEncoding):
 
     def project_rotate_store(self, h, w_qkv, qkv, ctx, cache, n_heads, n_kv_heads, head_dim) -> bool:
         """Few rows in bfloat16 with full rotary: the projection kernel rotates and writes the cache."""
-        from .base import DeferredRows
-        from .linear import FEW_ROWS
         rt = self.runtime
         row_factor = None
         if isinstance(h, DeferredRows):
