@@ -137,7 +137,8 @@ def run_mixed(args):
     pool = sum((l + gen + args.page_size - 1) // args.page_size * args.page_size for l in lens) + 64 * args.page_size
     engine, conf = build_engine(args.layers, pool, n_req, args.page_size)
     if not args.no_tune:
-        engine.tune_library_products([b for b in (n_req,) if b > 16])
+        # the two step sizes that recur: a full token budget, and one token of every request
+        engine.tune_library_products([budget] + [b for b in (n_req,) if b > 16])
     g = torch.Generator().manual_seed(1)
     prompts = [torch.randint(0, conf.vocab_size, (l,), generator=g).tolist() for l in lens]
 
