@@ -477,7 +477,7 @@ def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page):
 
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 200, 344, 331), (8, 2304, 2304, 6912), (16, 96, 509, 64), (5, 4096, 130, 50),
-                                      (3, 1536, 3840, 1000)])
+                                      (3, 1536, 3840, 1000), (7, 304, 8264, 130), (16, 512, 16384, 96)])
 def test_norm_split_over_two_products(M, N, K, N2):
     """Residual add + RMS norm between two products, split over them: the first product's
     epilogue adds to the stream and stores x * w with sums of squares; the second applies the
