@@ -65,10 +65,10 @@ struct NormFuse {
     float* ss_out;             // [gridDim.x, 16]
 };
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI>
+template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI, bool OWN_K = false>
 __global__ void __launch_bounds__(WPB * 64)
 gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C,
-                    int M, int N, int K, int lda, int ldw, int ldc, float alpha, RopeEpilogue rope, NormFuse nf, int own_k) {
+                    int M, int N, int K, int lda, int ldw, int ldc, float alpha, RopeEpilogue rope, NormFuse nf) {
     constexpr bool CSWIGLU = (EPI == 1);
     constexpr bool CROPE = (EPI == 2);
     constexpr bool CRESID = (EPI == 3);
@@ -151,13 +151,13 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     }
 
     // k-steps of 32 are dealt to the waves in turn; UNROLL steps are loaded before any is used.
-    // own_k (for long rows): a wave owns a contiguous run of steps instead, so that it walks
+    // OWN_K (for long rows): a wave owns a contiguous run of steps instead, so that it walks
     // UNROLL * 64 bytes of every row at a time and one stretch of each row overall.
     const int nsteps = (K + 31) >> 5;
-    const int spw = ((nsteps + WPB - 1) / WPB + UNROLL - 1) / UNROLL * UNROLL;      // own_k: steps per wave
-    const int s_begin = own_k ? wave * spw : wave;
-    const int s_end = own_k ? ((wave + 1) * spw < nsteps ? (wave + 1) * spw : nsteps) : nsteps;
-    const int s_stride = own_k ? 1 : WPB;                    // between the UNROLL steps of one iteration
+    const int spw = ((nsteps + WPB - 1) / WPB + UNROLL - 1) / UNROLL * UNROLL;      // OWN_K: steps per wave
+    const int s_begin = OWN_K ? wave * spw : wave;
+    const int s_end = OWN_K ? ((wave + 1) * spw < nsteps ? (wave + 1) * spw : nsteps) : nsteps;
+    constexpr int s_stride = OWN_K ? 1 : WPB;                // between the UNROLL steps of one iteration
     for (int s0 = s_begin; s0 < s_end; s0 += s_stride * UNROLL) {
         v4s wlo[UNROLL][NT], whi[UNROLL][NT], alo[UNROLL][MT], ahi[UNROLL][MT];
 #pragma unroll
@@ -314,17 +314,16 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         }
 }
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0>
+template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0, bool OWN_K = false>
 static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
-                        int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream, int blocks = 0,
-                        int own_k = 0) {
+                        int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream, int blocks = 0) {
     dim3 grid(blocks > 0 ? blocks : (N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf, own_k);
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI, OWN_K>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, EPI>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf, own_k);
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, EPI, OWN_K>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
 }
 
 // The gate/up projection with the activation in its epilogue: W [N, K] = [gate; up], C [M, N/2].
@@ -336,10 +335,10 @@ static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int
     dim3 grid(blocks, (M + 15) / 16), block(WPB * 64);
     if (aligned)
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, true, 1>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf, 0);
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
     else
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, false, 1>), grid, block, 0, stream,
-                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf, 0);
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
 }
 
 // Compute units of the current device, asked once.
@@ -475,7 +474,7 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
         // a long K over few columns (the down projection) does better with fewer, longer waves (from a sweep)
         const int blocks = ic_gemm_nt_residual_parts(N);
         // rows of 16 KB and more: a wave owns one stretch of every row (8B shape's down projection: 36 -> 30 us)
-        if (K >= kOwnKFrom) launch_gemm<bf16, 1, 1, 16, 2, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks, 1);
+        if (K >= kOwnKFrom) launch_gemm<bf16, 1, 1, 16, 2, 3, true>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
         else if (K > 2 * N) launch_gemm<bf16, 1, 1, 8, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
         else launch_gemm<bf16, 1, 1, 16, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
         return ic_launch_status();
@@ -526,7 +525,7 @@ IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int
     dim3 grid(blocks, 1);
 #define IC_ROPE(WPB, UN, AL)                                                                             \
     hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, WPB, UN, AL, 2>), grid, dim3(WPB * 64), 0, stream, \
-                       (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf, 0)
+                       (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf)
     // 8 waves, 4 steps in flight: within 4 % of the best tiling at every shape swept, and it does not spill
     if (aligned) IC_ROPE(8, 4, true); else IC_ROPE(8, 4, false);
 #undef IC_ROPE
