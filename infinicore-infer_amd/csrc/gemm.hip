@@ -45,6 +45,7 @@ struct RopeEpilogue {
     void* kcache;              // [pages, nkvh, page_size, dh]
     void* vcache;
     int nh, nkvh, dh, page_size;
+    int rr;                    // weight rows per tile that are used: 16, 8 or 4 (few heads: smaller tiles make more blocks)
 };
 
 // A norm split over two products (M <= 16).  The product BEFORE the norm (EPI == 3) owns the
@@ -82,8 +83,9 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     // for its R columns of the N/2 wide output.  R need not be a multiple of 16: the launcher picks
     // the number of blocks so that they fill the chip in one round where 16-row tiles would need
     // a second, part-filled one.
-    // CROPE: W = [q heads; k heads; v heads] (rows of dh).  A block owns 16 rows j.. of one q or k
-    // head and the 16 rows j + dh/2.. that rotate with them, or 32 consecutive rows of a v head.
+    // CROPE: W = [q heads; k heads; v heads] (rows of dh).  A block owns rr (16, 8 or 4) rows j.. of one q
+    // or k head and the rr rows j + dh/2.. that rotate with them, or 2 rr consecutive rows of a v head; with
+    // rr < 16 the other rows of its two tiles repeat the last one and are dropped.
     constexpr int G = CSWIGLU ? NT / 2 : 1;
     const int NO = CSWIGLU ? N / 2 : N;                      // output columns
     const int sw_cols = CSWIGLU ? (NO + (int)gridDim.x - 1) / (int)gridDim.x : 0;
@@ -97,14 +99,14 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     int rope_head = 0, rope_j = 0;                           // CROPE: head and first index in the head
     bool rope_is_v = false;
     if (CROPE) {
-        const int half = rope.dh >> 1, pt = half >> 4, n_rot = (rope.nh + rope.nkvh) * pt;
+        const int half = rope.dh >> 1, pt = half / rope.rr, n_rot = (rope.nh + rope.nkvh) * pt;
         const int p = blockIdx.x;
-        if (p < n_rot) { rope_head = p / pt; rope_j = 16 * (p - rope_head * pt); }
+        if (p < n_rot) { rope_head = p / pt; rope_j = rope.rr * (p - rope_head * pt); }
         else {
-            const int vt = rope.dh >> 5, pv = p - n_rot;
+            const int vt = rope.dh / (2 * rope.rr), pv = p - n_rot;
             rope_is_v = true;
             rope_head = rope.nh + rope.nkvh + pv / vt;
-            rope_j = 32 * (pv % vt);
+            rope_j = 2 * rope.rr * (pv % vt);
         }
         n0 = rope_head * rope.dh + rope_j;
     }
@@ -113,8 +115,8 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
     for (int nt = 0; nt < NT; ++nt) {
         int base = CSWIGLU ? n0 + 16 * (nt % G) + (nt / G) * NO : n0 + 16 * nt;
-        if (CROPE && nt == 1 && !rope_is_v) base = n0 + (rope.dh >> 1);
-        const int lim = CSWIGLU ? (nt / G) * NO + sw_end : (CRESID ? rs_end : N);
+        if (CROPE) base = n0 + nt * (rope_is_v ? rope.rr : (rope.dh >> 1));
+        const int lim = CSWIGLU ? (nt / G) * NO + sw_end : (CRESID ? rs_end : (CROPE ? base + rope.rr : N));
         const int nrow = (base + r < lim) ? base + r : lim - 1;
         wp[nt] = W + (size_t)nrow * ldw + 8 * kq;
     }
@@ -248,6 +250,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
             v0[e] = to_f32(from_f32<TC>(alpha * a0));   // the projection is rounded to its type first, as when stored
             v1[e] = to_f32(from_f32<TC>(alpha * a1));
         }
+        if (4 * kq >= rope.rr) return;                  // rows of the tiles that repeat the last one
         const int half = rope.dh >> 1;
         const int slot = rope.slots[m];
         const int pg = slot >= 0 ? slot / rope.page_size : 0, off = slot >= 0 ? slot - pg * rope.page_size : 0;
@@ -257,7 +260,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
             const int kh = rope_head - rope.nh - rope.nkvh;
             TC* dst = (TC*)rope.vcache + (((size_t)pg * rope.nkvh + kh) * rope.page_size + off) * rope.dh;
 #pragma unroll
-            for (int e = 0; e < 4; ++e) { dst[jj + e] = from_f32<TC>(v0[e]); dst[jj + 16 + e] = from_f32<TC>(v1[e]); }
+            for (int e = 0; e < 4; ++e) { dst[jj + e] = from_f32<TC>(v0[e]); dst[jj + rope.rr + e] = from_f32<TC>(v1[e]); }
             return;
         }
         const float4 c = *reinterpret_cast<const float4*>(rope.cos_t + (size_t)rope.positions[m] * half + jj);
@@ -508,6 +511,14 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
 // dh a multiple of 32.  W: [(nh + 2 nkvh) * dh, K].
 IC_EXPORT int ic_gemm_qkv_rope_supported(int dtype, int dh) { return dtype == IC_BF16 && dh >= 32 && dh % 32 == 0; }
 
+// For tuning and tests: the used rows per tile of ic_gemm_qkv_rope (16, 8 or 4; 0: chosen from the number of heads).
+static int g_rope_tile_rows = 0;
+IC_EXPORT int ic_gemm_qkv_rope_tile_rows(int rows) {
+    if (rows != 0 && rows != 4 && rows != 8 && rows != 16) return IC_ERR_ARG;
+    g_rope_tile_rows = rows;
+    return IC_OK;
+}
+
 IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc,
                                const int* positions, const int* slots, const float* cos_t, const float* sin_t,
                                void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size,
@@ -517,11 +528,18 @@ IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int
     if (!ic_gemm_qkv_rope_supported(IC_BF16, dh)) return IC_ERR_UNSUPPORTED;
     if (((uintptr_t)cos_t & 15) || ((uintptr_t)sin_t & 15)) return IC_ERR_ARG;
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
-    const RopeEpilogue rope{positions, slots, cos_t, sin_t, kcache, vcache, nh, nkvh, dh, page_size};
+    // rows per tile: few heads make few blocks of 16 + 16 rows; tiles of 8 or 4 used rows make two or four times as
+    // many.  The unused rows still cost load cycles, so it pays only well below one block per compute unit
+    // (measured: 80 blocks on 256 units 7.6 -> 6.9 us with 8 rows; 144 blocks 16.1 -> 19.6, slower).
+    const int pairs16 = (nh + 2 * nkvh) * (dh / 32), cus = compute_units();
+    int rr = 16;
+    if (g_rope_tile_rows) rr = g_rope_tile_rows;
+    else if (5 * pairs16 < 2 * cus) rr = (6 * pairs16 <= cus) ? 4 : 8;
+    const RopeEpilogue rope{positions, slots, cos_t, sin_t, kcache, vcache, nh, nkvh, dh, page_size, rr};
     const int N = (nh + 2 * nkvh) * dh;
     NormFuse nf{};
     if (!norm_fuse_args(row_factor, nullptr, M, N, K, IC_BF16, 0, nf)) return IC_ERR_ARG;
-    const int blocks = (nh + nkvh) * (dh / 32) + nkvh * (dh / 32);
+    const int blocks = pairs16 * (16 / rr);
     dim3 grid(blocks, 1);
 #define IC_ROPE(WPB, UN, AL)                                                                             \
     hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, WPB, UN, AL, 2>), grid, dim3(WPB * 64), 0, stream, \

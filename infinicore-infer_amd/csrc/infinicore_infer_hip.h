@@ -74,6 +74,8 @@ int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, in
 // QKV projection of M <= 16 rows with rotary and cache write in the epilogue; row_factor nullable.
 int ic_gemm_qkv_rope_supported(int dtype, int dh);
 int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc, const int* positions, const int* slots, const float* cos_t, const float* sin_t, void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size, const IcRowFactor* row_factor, hipStream_t stream);
+// For tuning and tests: used weight rows per tile of ic_gemm_qkv_rope (16, 8 or 4; 0: chosen from the number of heads).
+int ic_gemm_qkv_rope_tile_rows(int rows);
 
 // ---- matmul_library.hip ------------------------------------------------------------------------------
 // The library (hipBLASLt) matrix product for many rows: C[M, N] = alpha * A[M, K] W[N, K]^T, bfloat16 operands with a

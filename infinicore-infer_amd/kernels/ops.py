@@ -402,6 +402,12 @@ def gemm_qkv_rope_supported(dtype, head_dim: int) -> bool:
         return False
 
 
+def gemm_qkv_rope_tile_rows(rows: int) -> None:
+    """For tuning and tests: weight rows per tile that gemm_qkv_rope uses (16, 8 or 4; 0: chosen from the number
+    of heads, so that few heads still make a block for every compute unit)."""
+    check(get_lib().ic_gemm_qkv_rope_tile_rows(int(rows)), "gemm_qkv_rope_tile_rows")
+
+
 def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads, n_kv_heads, head_dim, page_size,
                   row_factor=None):
     """For M <= 16 rows: qkv = a @ w^T with the rotary encoding and the cache write in the epilogue.

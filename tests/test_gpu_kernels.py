@@ -446,11 +446,13 @@ def test_gemm_nt_with_swiglu_output(cdtype, M, di, K):
 
 @pytest.mark.parametrize("M,nh,nkvh,dh,K,page", [(1, 4, 2, 32, 96, 16), (8, 6, 2, 64, 200, 16), (16, 3, 3, 64, 2304, 64),
                                                  (5, 4, 1, 128, 344, 32), (3, 36, 36, 64, 2304, 64)])
-def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page):
+@pytest.mark.parametrize("tile_rows", [0, 16, 8, 4])
+def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page, tile_rows):
     """The fused projection + rotary + cache write equals the plain product followed by the
-    rotary/cache-write kernel."""
+    rotary/cache-write kernel, with every number of used rows per tile (0: chosen from the heads)."""
     g = torch.Generator().manual_seed(31)
     ops = _ops()
+    ops.gemm_qkv_rope_tile_rows(tile_rows)
     H = (nh + 2 * nkvh) * dh
     h = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (torch.randn(H, K, generator=g) * 0.1).to(torch.bfloat16)
@@ -464,7 +466,10 @@ def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page):
     kc = torch.zeros(n_pages, nkvh, page, dh, dtype=torch.bfloat16, device=DEV)
     vc = torch.zeros_like(kc)
     qkv = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
-    ops.gemm_qkv_rope(h.to(DEV), w.to(DEV), qkv, pos.to(DEV), slots.to(DEV), cos, sin, kc, vc, nh, nkvh, dh, page)
+    try:
+        ops.gemm_qkv_rope(h.to(DEV), w.to(DEV), qkv, pos.to(DEV), slots.to(DEV), cos, sin, kc, vc, nh, nkvh, dh, page)
+    finally:
+        ops.gemm_qkv_rope_tile_rows(0)
     # the two-kernel path
     kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
     ref = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
