@@ -492,11 +492,11 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
         if (c_dtype == IC_F32) {
             if (one_round) launch_gemm_swiglu<float, 8, 2, 2>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream, blocks);
             else if (tiles < 300) launch_gemm_swiglu<float, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
-            else launch_gemm_swiglu<float, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
+            else launch_gemm_swiglu<float, 16, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
         } else {
             if (one_round) launch_gemm_swiglu<bf16, 8, 2, 2>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream, blocks);
             else if (tiles < 300) launch_gemm_swiglu<bf16, 8>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
-            else launch_gemm_swiglu<bf16, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);
+            else launch_gemm_swiglu<bf16, 16, 4>(A, W, C, M, N, K, lda, ldw, ldc, aligned, nf, stream);   // many tiles (8B shape): 61 -> 55 us against 4 waves
         }
         return ic_launch_status();
     }
