@@ -474,11 +474,12 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
     if (!norm_fuse_args(row_factor, tail, M, N, K, c_dtype, ic_gemm_nt_residual_parts(N), nf)) return IC_ERR_ARG;
     const bool aligned = (lda % 8 == 0) && (ldw % 8 == 0) && (((uintptr_t)A & 15) == 0) && (((uintptr_t)W & 15) == 0);
     if (c_mode == 2) {
-        // a long K over few columns (the down projection) does better with fewer, longer waves (from a sweep)
+        // 16 waves a block throughout; up to 4 rows 4 k-steps in flight, above that 2 (from a sweep over the O and
+        // down projections of the 1B..8B shapes with one block per compute unit)
         const int blocks = ic_gemm_nt_residual_parts(N);
         // rows of 16 KB and more: a wave owns one stretch of every row (8B shape's down projection: 36 -> 30 us)
         if (K >= kOwnKFrom) launch_gemm<bf16, 1, 1, 16, 2, 3, true>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
-        else if (K > 2 * N) launch_gemm<bf16, 1, 1, 8, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
+        else if (M > 4) launch_gemm<bf16, 1, 1, 16, 2, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
         else launch_gemm<bf16, 1, 1, 16, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
         return ic_launch_status();
     }
