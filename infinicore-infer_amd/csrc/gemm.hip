@@ -13,6 +13,7 @@
 // 16x16x16 layout (lane l): A[i = l%16][k = 4(l/16)..+3], B[k = 4(l/16)..+3][j = l%16],
 // D[i = 4(l/16) + e][j = l%16], e = 0..3.
 #include "common.h"
+#include <utility>
 
 typedef short v4s __attribute__((ext_vector_type(4)));
 typedef float v4f __attribute__((ext_vector_type(4)));
@@ -66,7 +67,26 @@ struct NormFuse {
     float* ss_out;             // [gridDim.x, 16]
 };
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI, bool OWN_K = false>
+// lane i of a row of 16 lanes takes the value of lane (i + S) % 16 (a DPP row rotation, no LDS)
+template <int S> __device__ __forceinline__ v4s row_from_above(v4s v) {
+    if constexpr (S % 16 == 0) return v;
+    else {
+        typedef int v2i __attribute__((ext_vector_type(2)));
+        const v2i a = __builtin_bit_cast(v2i, v);
+        v2i b;
+        b[0] = __builtin_amdgcn_update_dpp(0, a[0], 0x120 + (16 - S % 16), 0xf, 0xf, false);
+        b[1] = __builtin_amdgcn_update_dpp(0, a[1], 0x120 + (16 - S % 16), 0xf, 0xf, false);
+        return __builtin_bit_cast(v4s, b);
+    }
+}
+// step u of an iteration takes its token operand out of the register that was loaded for its group of AG steps
+template <int AG, int MP, int... Us>
+__device__ __forceinline__ void spread_token_operand(const v4s* glo, const v4s* ghi, v4s (*alo)[1], v4s (*ahi)[1],
+                                                     std::integer_sequence<int, Us...>) {
+    ((alo[Us][0] = row_from_above<(Us % AG) * MP>(glo[Us / AG]), ahi[Us][0] = row_from_above<(Us % AG) * MP>(ghi[Us / AG])), ...);
+}
+
+template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI, bool OWN_K = false, int AG = 1>
 __global__ void __launch_bounds__(WPB * 64)
 gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C,
                     int M, int N, int K, int lda, int ldw, int ldc, float alpha, RopeEpilogue rope, NormFuse nf) {
@@ -172,15 +192,36 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
                 else { wlo[u][nt] = v4s{0, 0, 0, 0}; whi[u][nt] = wlo[u][nt]; }
             }
         }
+        if constexpr (AG == 1) {
 #pragma unroll
-        for (int u = 0; u < UNROLL; ++u) {
-            const int kk = 32 * (s0 + u * s_stride);
-            const int valid = (s0 + u * s_stride < s_end) ? K - kk - 8 * kq : 0;
+            for (int u = 0; u < UNROLL; ++u) {
+                const int kk = 32 * (s0 + u * s_stride);
+                const int valid = (s0 + u * s_stride < s_end) ? K - kk - 8 * kq : 0;
 #pragma unroll
-            for (int mt = 0; mt < MT; ++mt) {
-                if (valid > 0) load8<ALIGNED>(ap[mt] + kk, valid, alo[u][mt], ahi[u][mt]);
-                else { alo[u][mt] = v4s{0, 0, 0, 0}; ahi[u][mt] = alo[u][mt]; }
+                for (int mt = 0; mt < MT; ++mt) {
+                    if (valid > 0) load8<ALIGNED>(ap[mt] + kk, valid, alo[u][mt], ahi[u][mt]);
+                    else { alo[u][mt] = v4s{0, 0, 0, 0}; ahi[u][mt] = alo[u][mt]; }
+                }
             }
+        } else {
+            // Up to 16 / AG rows (MT == 1): one load serves AG steps.  Lane r of a row of 16 loads token row
+            // r % MP of step r / MP; step t's operand is then that register rotated down by t * MP lanes
+            // (the columns from MP on hold other steps' rows and are never stored).  The cost of the token
+            // operand is the number of its load instructions, not its bytes.
+            static_assert(AG == 1 || (MT == 1 && UNROLL % AG == 0 && 16 % AG == 0), "grouped token loads");
+            constexpr int MP = 16 / AG;
+            v4s glo[UNROLL / AG], ghi[UNROLL / AG];
+            const int gt = r / MP, gm = r % MP;
+            const uint16_t* gp = A + (size_t)((m0 + gm < M) ? m0 + gm : M - 1) * lda + 8 * kq;
+#pragma unroll
+            for (int g = 0; g < UNROLL / AG; ++g) {
+                const int st = s0 + (g * AG + gt) * s_stride;
+                const int kk = 32 * st;
+                const int valid = (st < s_end && m0 + gm < M) ? K - kk - 8 * kq : 0;
+                if (valid > 0) load8<ALIGNED>(gp + kk, valid, glo[g], ghi[g]);
+                else { glo[g] = v4s{0, 0, 0, 0}; ghi[g] = glo[g]; }
+            }
+            spread_token_operand<AG, MP>(glo, ghi, alo, ahi, std::make_integer_sequence<int, UNROLL>{});
         }
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
@@ -317,15 +358,15 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         }
 }
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0, bool OWN_K = false>
+template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0, bool OWN_K = false, int AG = 1>
 static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
                         int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream, int blocks = 0) {
     dim3 grid(blocks > 0 ? blocks : (N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
     if (aligned)
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI, OWN_K>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI, OWN_K, AG>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
     else
-        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, EPI, OWN_K>), grid, block, 0, stream,
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, false, EPI, OWN_K, AG>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
 }
 
@@ -336,7 +377,11 @@ static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int
                                int ldc, bool aligned, const NormFuse& nf, hipStream_t stream, int blocks = 0) {
     if (blocks <= 0) blocks = (N / 2 + 16 * G - 1) / (16 * G);
     dim3 grid(blocks, (M + 15) / 16), block(WPB * 64);
-    if (aligned)
+    constexpr int AG = (UN % 4 == 0) ? 4 : 2;                // up to 4 rows one token load serves AG k-steps
+    if (aligned && M <= 4 && sizeof(TC) == 2)
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, true, 1, false, AG>), grid, block, 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
+    else if (aligned)
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, true, 1>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
     else
@@ -478,9 +523,13 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
         // down projections of the 1B..8B shapes with one block per compute unit)
         const int blocks = ic_gemm_nt_residual_parts(N);
         // rows of 16 KB and more: a wave owns one stretch of every row (8B shape's down projection: 36 -> 30 us)
-        if (K >= kOwnKFrom) launch_gemm<bf16, 1, 1, 16, 2, 3, true>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
-        else if (M > 4) launch_gemm<bf16, 1, 1, 16, 2, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
-        else launch_gemm<bf16, 1, 1, 16, 4, 3>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks);
+        // up to 8 (4) rows one load of the token operand serves 2 (4) k-steps
+#define IC_RES(UN, OWN, AG) launch_gemm<bf16, 1, 1, 16, UN, 3, OWN, AG>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream, blocks)
+        if (K >= kOwnKFrom) { if (M <= 8) IC_RES(2, true, 2); else IC_RES(2, true, 1); }
+        else if (M > 8) IC_RES(2, false, 1);
+        else if (M > 4) IC_RES(2, false, 2);
+        else IC_RES(4, false, 4);
+#undef IC_RES
         return ic_launch_status();
     }
     if (c_mode == 1) {
@@ -546,7 +595,11 @@ IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int
     hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, WPB, UN, AL, 2>), grid, dim3(WPB * 64), 0, stream, \
                        (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf)
     // 8 waves, 4 steps in flight: within 4 % of the best tiling at every shape swept, and it does not spill
-    if (aligned) IC_ROPE(8, 4, true); else IC_ROPE(8, 4, false);
+    if (aligned && M <= 4)                                  // one token load serves the 4 k-steps of an iteration
+        hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, 8, 4, true, 2, false, 4>), grid, dim3(8 * 64), 0, stream,
+                           (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf);
+    else if (aligned) IC_ROPE(8, 4, true);
+    else IC_ROPE(8, 4, false);
 #undef IC_ROPE
     return ic_launch_status();
 }
