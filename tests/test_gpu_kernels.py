@@ -431,7 +431,7 @@ def test_sampling_distribution():
 
 @pytest.mark.parametrize("cdtype", DT)
 @pytest.mark.parametrize("M,di,K", [(1, 344, 200), (8, 5760, 2304), (16, 256, 96), (5, 130, 100), (3, 3840, 1536),
-                                    (5, 8400, 136)])       # the last: more tiles than one round of blocks takes
+                                    (5, 8400, 136), (2, 8400, 2048)])    # the last two: more tiles than one round of blocks takes
 def test_gemm_nt_with_swiglu_output(cdtype, M, di, K):
     """The gate/up projection with the activation in its epilogue equals the plain product
     followed by the SwiGLU kernel."""
