@@ -39,7 +39,7 @@ union Frag8 {
     bf16x8 v;
 };
 
-template <int DH, bool STAGED, int GROUPS>
+template <int DH, bool STAGED, int GROUPS, bool PAGE64>
 __global__ void __launch_bounds__(256 * GROUPS, (GROUPS == 1 && DH <= 64) ? 3 : 2)
 attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                          const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
@@ -122,7 +122,21 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     // thread -> (key, octet) for K (octets along lanes: whole rows per wave) and
     // (octet, key) for V (keys along lanes: conflict-free transposed stores)
     uint4 kreg[NL], vreg[NL];
+    // PAGE64 (pages of 64 tokens and more): a 64-key tile lies in one page, so a step needs one page
+    // lookup per tile and every load is that tile's first row plus an offset the thread keeps.
+    constexpr int KPI = kPfThreads / (DH / 8);                // keys one pass of K loads covers (<= 64)
+    static_assert(KPI <= kPfKeys && kPfKeys % KPI == 0 && kPfThreads % STEP == 0, "a pass of loads stays inside a tile");
+    const int vkey = tid % STEP;                              // the key (within the step) of this thread's V loads
     auto fetch = [&](int kt) {
+        size_t tile_row[GROUPS];                              // PAGE64: element offset of each tile's first row
+        if (PAGE64) {
+#pragma unroll
+            for (int t = 0; t < GROUPS; ++t) {
+                const int k0 = kt + kPfKeys * t;
+                const int k0c = (k0 <= last_key) ? k0 : last_key;     // a tile beyond the end is not loaded at all
+                tile_row[t] = (size_t)page_of(k0c) * page_stride + (size_t)(k0 & page_mask) * DH;
+            }
+        }
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
             const int idx = tid + i * kPfThreads;
@@ -131,8 +145,12 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                 const int ka = kt + key;
                 kreg[i] = make_uint4(0, 0, 0, 0);
                 if (ka <= last_key && ka >= first_key) {
-                    const int pg = page_of(ka), off = ka & page_mask;
-                    kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)pg * page_stride + (size_t)off * DH + oct * 8);
+                    if (PAGE64) {
+                        kreg[i] = *reinterpret_cast<const uint4*>(kbase + tile_row[(i * KPI) / kPfKeys] + (size_t)(key % kPfKeys) * DH + oct * 8);
+                    } else {
+                        const int pg = page_of(ka), off = ka & page_mask;
+                        kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)pg * page_stride + (size_t)off * DH + oct * 8);
+                    }
                 }
             }
             {
@@ -140,8 +158,12 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                 const int ka = kt + key;
                 vreg[i] = make_uint4(0, 0, 0, 0);
                 if (ka <= last_key && ka >= first_key) {
-                    const int pg = page_of(ka), off = ka & page_mask;
-                    vreg[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)pg * page_stride + (size_t)off * DH + oct * 8);
+                    if (PAGE64) {
+                        vreg[i] = *reinterpret_cast<const uint4*>(vbase + tile_row[GROUPS == 1 ? 0 : vkey / kPfKeys] + (size_t)(vkey % kPfKeys) * DH + oct * 8);
+                    } else {
+                        const int pg = page_of(ka), off = ka & page_mask;
+                        vreg[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)pg * page_stride + (size_t)off * DH + oct * 8);
+                    }
                 }
             }
         }
@@ -325,11 +347,13 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
     }
     const bool two_groups = groups ? groups == 2 : 4LL * nh * n_tiles < 11LL * cus;
     dim3 grid((unsigned)nh * (unsigned)n_tiles);
-#define IC_PF_LAUNCH(DD, ST, GG)                                                                                   \
-    hipLaunchKernelGGL((attn_prefill_mfma_kernel<DD, ST, GG>), grid, dim3(256 * GG), 0, stream, (const uint16_t*)q, \
+    const bool page64 = page_size >= kPfKeys;            // (a power of two) a 64-key tile lies in one page
+#define IC_PF_LAUNCH(DD, ST, GG, PP)                                                                                   \
+    hipLaunchKernelGGL((attn_prefill_mfma_kernel<DD, ST, GG, PP>), grid, dim3(256 * GG), 0, stream, (const uint16_t*)q, \
                        q_stride, (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
                        block_tables, bt_stride, (const int4*)tiles, n_tiles, nh, nkvh, page_shift, sl2, window)
-#define IC_PF_GROUPS(DD, ST) do { if (two_groups) IC_PF_LAUNCH(DD, ST, 2); else IC_PF_LAUNCH(DD, ST, 1); } while (0)
+#define IC_PF_GROUPS(DD, ST) do { if (two_groups) { if (page64) IC_PF_LAUNCH(DD, ST, 2, true); else IC_PF_LAUNCH(DD, ST, 2, false); } \
+                                  else { if (page64) IC_PF_LAUNCH(DD, ST, 1, true); else IC_PF_LAUNCH(DD, ST, 1, false); } } while (0)
     if (dh == 64) { if (staged) IC_PF_GROUPS(64, true); else IC_PF_GROUPS(64, false); }
     else if (dh == 128) { if (staged) IC_PF_GROUPS(128, true); else IC_PF_GROUPS(128, false); }
 #undef IC_PF_GROUPS
