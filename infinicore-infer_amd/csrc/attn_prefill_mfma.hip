@@ -6,9 +6,11 @@
 // the two groups take the even and the odd key tiles of 64 and are merged through LDS at the
 // end: the longest query tile of a prompt, which sets the kernel's time when there are few
 // blocks, then walks half as many key tiles.  With many blocks GROUPS == 1 keeps more of them
-// resident and is faster.  Keys and values come through LDS, 64 * GROUPS keys a step (values
-// transposed on the way in); the next step is already on its way from memory while the
-// current one is used.  Scores
+// resident and is faster.  Keys and values come through LDS as rows, 64 * GROUPS keys a step; the
+// next step is already on its way from memory while the current one is used.  The V^T operand is
+// read with ds_read_b64_tr_b16, which transposes 16-bit elements across the lanes of a 16-lane
+// group on the way out of LDS (lane 16G + i receives, for e = 0..3, element i % 4 of the 8-byte
+// chunk that lane 16G + i / 4 + 4e pointed at).  Scores
 // are computed transposed, S^T = K Q^T, with v_mfma_f32_32x32x16_bf16: every
 // lane then holds 32 keys of ONE query, so the running softmax needs a single
 // cross-lane step, and the probabilities are already laid out as the B operand
@@ -26,6 +28,7 @@
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
 typedef float v8f __attribute__((ext_vector_type(8)));
+typedef short tr_v4s __attribute__((ext_vector_type(4)));
 
 constexpr int kPfWaveThreads = 256;   // four waves own the 128 rows of a query tile
 constexpr int kPfRows = 128;      // query rows per block
@@ -47,17 +50,16 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                          int n_tiles, int nh, int nkvh, int page_shift, float scale_log2e, int window) {
     constexpr int NC = DH / 16;           // 16-wide chunks of the head dimension
     constexpr int ND = DH / 32;           // 32-row tiles of O^T
-    constexpr int KS = DH + kPfPad;       // row stride of Ks (elements)
-    constexpr int VS = kPfKeys + kPfPad;  // row stride of Vt
+    constexpr int KS = DH + kPfPad;       // row stride of Ks and Vs (elements)
     constexpr int kPfThreads = kPfWaveThreads * GROUPS;
     constexpr int STEP = kPfKeys * GROUPS;                 // keys staged per step
     constexpr int NL = STEP * (DH / 8) / kPfThreads;       // 16-byte loads per thread per plane and step
-    constexpr int KT = kPfKeys * KS, VT = DH * VS;         // elements of one group's K and V^T tile
+    constexpr int KT = kPfKeys * KS, VT = KT;              // elements of one group's K and V tile
     constexpr int MERGE_F = 2 + ND * 16;                   // floats a lane hands over at the end
     static_assert(GROUPS == 1 || sizeof(uint16_t) * GROUPS * (KT + VT) >= sizeof(float) * 256 * MERGE_F, "merge buffer fits in the tiles");
     __shared__ __attribute__((aligned(16))) uint16_t tilebuf[GROUPS * (KT + VT)];
     uint16_t* const Ks_all = tilebuf;                      // [group][key][KS]
-    uint16_t* const Vt_all = tilebuf + GROUPS * KT;     // [group][dim][VS]
+    uint16_t* const Vs_all = tilebuf + GROUPS * KT;     // [group][key][KS]
 
     __shared__ int pages[kPfMaxPages];
 
@@ -119,14 +121,12 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     const uint16_t* vbase = vcache + (size_t)kvh * head_stride;
     const size_t page_stride = (size_t)nkvh * head_stride;
 
-    // thread -> (key, octet) for K (octets along lanes: whole rows per wave) and
-    // (octet, key) for V (keys along lanes: conflict-free transposed stores)
+    // thread -> (key, octet), octets along lanes: a wave loads and stores whole rows of K and of V
     uint4 kreg[NL], vreg[NL];
     // PAGE64 (pages of 64 tokens and more): a 64-key tile lies in one page, so a step needs one page
     // lookup per tile and every load is that tile's first row plus an offset the thread keeps.
     constexpr int KPI = kPfThreads / (DH / 8);                // keys one pass of K loads covers (<= 64)
-    static_assert(KPI <= kPfKeys && kPfKeys % KPI == 0 && kPfThreads % STEP == 0, "a pass of loads stays inside a tile");
-    const int vkey = tid % STEP;                              // the key (within the step) of this thread's V loads
+    static_assert(KPI <= kPfKeys && kPfKeys % KPI == 0, "a pass of loads stays inside a tile");
     auto fetch = [&](int kt) {
         size_t tile_row[GROUPS];                              // PAGE64: element offset of each tile's first row
         if (PAGE64) {
@@ -144,26 +144,13 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                 const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
                 const int ka = kt + key;
                 kreg[i] = make_uint4(0, 0, 0, 0);
-                if (ka <= last_key && ka >= first_key) {
-                    if (PAGE64) {
-                        kreg[i] = *reinterpret_cast<const uint4*>(kbase + tile_row[(i * KPI) / kPfKeys] + (size_t)(key % kPfKeys) * DH + oct * 8);
-                    } else {
-                        const int pg = page_of(ka), off = ka & page_mask;
-                        kreg[i] = *reinterpret_cast<const uint4*>(kbase + (size_t)pg * page_stride + (size_t)off * DH + oct * 8);
-                    }
-                }
-            }
-            {
-                const int oct = idx / STEP, key = idx - oct * STEP;
-                const int ka = kt + key;
                 vreg[i] = make_uint4(0, 0, 0, 0);
                 if (ka <= last_key && ka >= first_key) {
-                    if (PAGE64) {
-                        vreg[i] = *reinterpret_cast<const uint4*>(vbase + tile_row[GROUPS == 1 ? 0 : vkey / kPfKeys] + (size_t)(vkey % kPfKeys) * DH + oct * 8);
-                    } else {
-                        const int pg = page_of(ka), off = ka & page_mask;
-                        vreg[i] = *reinterpret_cast<const uint4*>(vbase + (size_t)pg * page_stride + (size_t)off * DH + oct * 8);
-                    }
+                    size_t off;
+                    if (PAGE64) off = tile_row[(i * KPI) / kPfKeys] + (size_t)(key % kPfKeys) * DH + oct * 8;
+                    else off = (size_t)page_of(ka) * page_stride + (size_t)(ka & page_mask) * DH + oct * 8;
+                    kreg[i] = *reinterpret_cast<const uint4*>(kbase + off);
+                    vreg[i] = *reinterpret_cast<const uint4*>(vbase + off);
                 }
             }
         }
@@ -172,24 +159,15 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
             const int idx = tid + i * kPfThreads;
-            {
-                const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
-                *reinterpret_cast<uint4*>(&Ks_all[(key / kPfKeys) * KT + (key % kPfKeys) * KS + oct * 8]) = kreg[i];
-            }
-            {
-                const int oct = idx / STEP, key = idx - oct * STEP;
-                const uint4 v = vreg[i];
-                uint16_t* vp = &Vt_all[(key / kPfKeys) * VT + (oct * 8) * VS + (key % kPfKeys)];
-                vp[0 * VS] = (uint16_t)(v.x & 0xffff); vp[1 * VS] = (uint16_t)(v.x >> 16);
-                vp[2 * VS] = (uint16_t)(v.y & 0xffff); vp[3 * VS] = (uint16_t)(v.y >> 16);
-                vp[4 * VS] = (uint16_t)(v.z & 0xffff); vp[5 * VS] = (uint16_t)(v.z >> 16);
-                vp[6 * VS] = (uint16_t)(v.w & 0xffff); vp[7 * VS] = (uint16_t)(v.w >> 16);
-            }
+            const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
+            const int at = (key / kPfKeys) * KT + (key % kPfKeys) * KS + oct * 8;
+            *reinterpret_cast<uint4*>(&Ks_all[at]) = kreg[i];
+            *reinterpret_cast<uint4*>(&Vs_all[at]) = vreg[i];
         }
     };
 
     const uint16_t* const Ks = Ks_all + grp * KT;
-    const uint16_t* const Vt = Vt_all + grp * VT;
+    const uint16_t* const Vs = Vs_all + grp * VT;
     const int kt0 = (first_key / kPfKeys) * kPfKeys;
     fetch(kt0);
     for (int kb = kt0; kb <= last_key; kb += STEP) {
@@ -266,10 +244,12 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             const bf16x8 b = __builtin_convertvector(pf, bf16x8);
 #pragma unroll
             for (int dt = 0; dt < ND; ++dt) {
-                const uint16_t* vp = &Vt[(32 * dt + lq) * VS + 16 * kc + 4 * half];
+                // this lane's chunk: key 16 kc + 4 half + (l % 16) / 4 (and 8 keys on), dims 32 dt + 16 (l / 16 % 2) + 4 (l % 4) ..+3;
+                // what comes back is dim 32 dt + lq of keys 16 kc + 4 half + e (and 8 keys on), e = 0..3
+                const uint16_t* vp = &Vs[(16 * kc + 4 * half + ((lane & 15) >> 2)) * KS + 32 * dt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)];
                 Frag8 a;
-                a.h[0] = *reinterpret_cast<const uint2*>(vp);
-                a.h[1] = *reinterpret_cast<const uint2*>(vp + 8);
+                a.h[0] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)vp));
+                a.h[1] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)(vp + 8 * KS)));
                 oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b, oacc[dt], 0, 0, 0);
             }
         }
