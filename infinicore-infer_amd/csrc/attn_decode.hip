@@ -295,11 +295,12 @@ attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __res
 // 32-dim chunk).  A lane then holds 4+4 keys of ONE head (l%16), so the running softmax needs two
 // cross-lane steps.  O^T = V^T P^T: P^T is already the B operand (slot (l/16, e) stands for key
 // 4(l/16) + e of the first 16 keys for e < 4, of the second 16 for e >= 4); V goes through LDS
-// (written as rows, read as columns).  16x16x32 layout: A[i = l%16][k = 8(l/16)..+7],
+// (written as rows, read as columns with ds_read_b64_tr_b16).  16x16x32 layout: A[i = l%16][k = 8(l/16)..+7],
 // B[k = 8(l/16)..+7][j = l%16], D[i = 4(l/16) + e][j = l%16].
 typedef __bf16 gq_bf16x8 __attribute__((ext_vector_type(8)));
 typedef float gq_v4f __attribute__((ext_vector_type(4)));
 typedef float gq_v8f __attribute__((ext_vector_type(8)));
+typedef short gq_v4s __attribute__((ext_vector_type(4)));
 constexpr int kGqaKeys = 32;
 
 union GqFrag {
@@ -459,15 +460,17 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
             const gq_bf16x8 pb = __builtin_convertvector(pf, gq_bf16x8);
 
             // ---- O^T += V^T P^T ----------------------------------------------------------------
-            const uint16_t* vrow = &Vs[wave][(4 * lg) * VS + lr];
+            // V^T operand by transposing LDS reads: lane 16 G + i receives, for e = 0..3, element i % 4 of the
+            // 8-byte chunk that lane 16 G + i / 4 + 4 e pointed at; this lane points at key 4 lg + lr / 4 (and 16
+            // keys on), dims 16 c + 4 (lr % 4) ..+3, and gets dim 16 c + lr of keys 4 lg + e (and 16 keys on)
+            const uint16_t* vrow = &Vs[wave][(4 * lg + (lr >> 2)) * VS + 4 * (lr & 3)];
 #pragma unroll
             for (int c = 0; c < ND; ++c) {
                 GqFrag a;
+                const gq_v4s lo = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gq_v4s __attribute__((address_space(3)))*)(vrow + 16 * c));
+                const gq_v4s hi = __builtin_amdgcn_ds_read_tr16_b64_v4i16((gq_v4s __attribute__((address_space(3)))*)(vrow + 16 * VS + 16 * c));
 #pragma unroll
-                for (int e = 0; e < 4; ++e) {
-                    a.h[e] = vrow[e * VS + 16 * c];
-                    a.h[4 + e] = vrow[(16 + e) * VS + 16 * c];
-                }
+                for (int e = 0; e < 4; ++e) { a.h[e] = (uint16_t)lo[e]; a.h[4 + e] = (uint16_t)hi[e]; }
                 oacc[c] *= corr;
                 oacc[c] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(a.v, pb, oacc[c], 0, 0, 0);
             }
