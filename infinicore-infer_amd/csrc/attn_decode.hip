@@ -249,39 +249,50 @@ attn_decode_split_kernel(const T* __restrict__ q, int q_stride,
 }
 
 // Grid (tokens * heads), four waves.  Lane s of every wave holds split s (at most 64 splits): the
-// weights exp(m_s - max) come from one wave reduction.  Thread (d, g) then sums output dim d over
-// the splits g, g + G, .. (G = 256 / dh groups) with independent loads, and the groups meet in LDS:
-// with many splits (few kv heads, few requests) one wave alone would walk them one after the other.
+// weights exp(m_s - max) come from one wave reduction.  Thread (d, g) sums output dim d over
+// the splits g, g + G, .. (G = 256 / DH groups, CNT = ceil(splits / G) of them a thread), and the
+// groups meet in LDS: with many splits (few kv heads, few requests) one wave alone would walk them
+// one after the other.  The partial sums are loaded first, without condition (a slot beyond the
+// splits reads the last split and is not added): they do not wait for the weights, so the kernel
+// is one round trip to memory, not two.
 constexpr int kRedThreads = 256;
-template <typename T>
+template <typename T, int DH, int CNT>
 __global__ void __launch_bounds__(kRedThreads)
 attn_decode_reduce_kernel(const float* __restrict__ part_acc, const float* __restrict__ part_ml,
                           const int* __restrict__ tok_list, T* __restrict__ out,
-                          int out_stride, int nh, int dh, int nsplit) {
+                          int out_stride, int nh, int nsplit) {
+    constexpr int G = kRedThreads / DH;
+    static_assert(kRedThreads % DH == 0, "every thread has a (dim, group) place");
     __shared__ float wgt[64];
     __shared__ float grp[kRedThreads];
     const int n = blockIdx.x / nh, h = blockIdx.x % nh, tid = threadIdx.x, lane = tid & 63;
-    const int t = tok_list ? tok_list[n] : n;
     const size_t base = ((size_t)n * nh + h) * nsplit;
-    float ms = -INFINITY, ls = 0.f;
-    if (lane < nsplit) { ms = part_ml[(base + lane) * 2]; ls = part_ml[(base + lane) * 2 + 1]; }
+    const int g = tid / DH, d = tid - g * DH;
+    float pa[CNT];
+#pragma unroll
+    for (int i = 0; i < CNT; ++i) {
+        const int s = (g + i * G < nsplit) ? g + i * G : nsplit - 1;
+        pa[i] = part_acc[(base + s) * DH + d];
+    }
+    const int ls_i = (lane < nsplit) ? lane : nsplit - 1;
+    float ms = part_ml[(base + ls_i) * 2], ls = part_ml[(base + ls_i) * 2 + 1];
+    const int t = tok_list ? tok_list[n] : n;
+    if (lane >= nsplit) { ms = -INFINITY; ls = 0.f; }
     const float mm = wave_max(ms);
     const float w = (ms == -INFINITY) ? 0.f : expf(ms - mm);
     const float inv = 1.0f / wave_sum(ls * w);
     if (tid < 64) wgt[lane] = w;
     __syncthreads();
-    // dh <= 256: G >= 1 groups of dh threads
-    const int G = kRedThreads / dh, g = tid / dh, d = tid - g * dh;
     float a = 0.f;
-    if (g < G) {
-#pragma unroll 8
-        for (int s = g; s < nsplit; s += G) a += part_acc[(base + s) * dh + d] * wgt[s];
-    }
+#pragma unroll
+    for (int i = 0; i < CNT; ++i)
+        if (g + i * G < nsplit) a += pa[i] * wgt[g + i * G];
     grp[tid] = a;
     __syncthreads();
-    if (tid < dh) {
-        for (int j = 1; j < G; ++j) a += grp[j * dh + tid];
-        out[(size_t)t * out_stride + (size_t)h * dh + tid] = from_f32<T>(a * inv);
+    if (tid < DH) {
+#pragma unroll
+        for (int j = 1; j < G; ++j) a += grp[j * DH + tid];
+        out[(size_t)t * out_stride + (size_t)h * DH + tid] = from_f32<T>(a * inv);
     }
 }
 
@@ -536,8 +547,16 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
 #undef IC_DEC_LAUNCH
     int st = ic_launch_status();
     if (st || nsplit == 1) return st;
-    hipLaunchKernelGGL(attn_decode_reduce_kernel<T>, dim3(n_tok * nh), dim3(kRedThreads), 0, stream, part_acc, part_ml,
-                       tok_list, (T*)out, out_stride, nh, DH, nsplit);
+    const int per_thread = (nsplit + kRedThreads / DH - 1) / (kRedThreads / DH);    // splits a thread of the second pass sums
+#define IC_RED_LAUNCH(CNT)                                                                                      \
+    hipLaunchKernelGGL((attn_decode_reduce_kernel<T, DH, CNT>), dim3(n_tok * nh), dim3(kRedThreads), 0, stream, \
+                       part_acc, part_ml, tok_list, (T*)out, out_stride, nh, nsplit)
+    if (per_thread <= 2) IC_RED_LAUNCH(2);
+    else if (per_thread <= 4) IC_RED_LAUNCH(4);
+    else if (per_thread <= 8) IC_RED_LAUNCH(8);
+    else if (per_thread <= 16) IC_RED_LAUNCH(16);
+    else IC_RED_LAUNCH(32);                             // 64 splits, two groups
+#undef IC_RED_LAUNCH
     return ic_launch_status();
 }
 

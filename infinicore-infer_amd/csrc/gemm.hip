@@ -9,6 +9,10 @@
 // 16 bytes of each A row tile, and feeds them to two v_mfma_f32_16x16x16_bf16
 // as A and B operands.  Both operands use the same lane->k mapping, so the
 // order of k inside a step does not matter.  The waves' partial sums meet in LDS.
+// Two variants of the walk over K: OWN_K gives each wave one contiguous run of
+// k-steps (long rows), and AG > 1 lets one load of the token operand serve AG
+// k-steps when at most 16 / AG rows are in use (the spare lanes carry the other
+// steps' data and a row rotation hands it over).
 //
 // 16x16x16 layout (lane l): A[i = l%16][k = 4(l/16)..+3], B[k = 4(l/16)..+3][j = l%16],
 // D[i = 4(l/16) + e][j = l%16], e = 0..3.

@@ -40,6 +40,7 @@ struct Plan {
     std::vector<hipblasLtMatmulHeuristicResult_t> candidates;   // [0] is the library's first choice
     int chosen = 0;
     bool all_listed = false;                                     // every algorithm of the library was appended
+    bool timed = false;                                          // `chosen` comes from timing on the device
 };
 
 std::mutex g_mu;
@@ -47,6 +48,35 @@ hipblasLtHandle_t g_handle = nullptr;
 std::unordered_map<Key, Plan, KeyHash> g_plans;
 
 hipDataType lt_type(int dtype) { return dtype == IC_BF16 ? HIP_R_16BF : HIP_R_32F; }
+
+// A product that was not timed itself takes the algorithm that timing chose for the same matrices at the
+// nearest row count within an eighth of its own, if the library accepts it for this shape: the steps of a
+// running batch have token counts near the budget that was timed, seldom exactly it.
+void borrow_from_neighbour(const Key& key, Plan& p, size_t workspace_bytes) {
+    const Plan* from = nullptr;
+    int dist = 0;
+    for (const auto& kv : g_plans) {
+        const Key& o = kv.first;
+        if (!kv.second.timed || kv.second.chosen == 0) continue;
+        if (o.a_dtype != key.a_dtype || o.c_dtype != key.c_dtype || o.N != key.N || o.K != key.K || o.lda != key.lda ||
+            o.ldw != key.ldw || o.ldc != key.ldc)
+            continue;
+        const int d = o.M > key.M ? o.M - key.M : key.M - o.M;
+        if (8 * d > o.M) continue;
+        if (!from || d < dist) { from = &kv.second; dist = d; }
+    }
+    if (!from) return;
+    hipblasLtMatmulHeuristicResult_t r = from->candidates[from->chosen];
+    const float one = 1.f, zero = 0.f;
+    size_t need = 0;
+    if (hipblaslt_ext::matmulIsAlgoSupported(g_handle, p.desc, &one, p.lw, p.la, &zero, p.lc, p.lc, r.algo, need) !=
+            HIPBLAS_STATUS_SUCCESS || need > workspace_bytes)
+        return;
+    r.workspaceSize = need;
+    r.state = HIPBLAS_STATUS_SUCCESS;
+    p.candidates.push_back(r);
+    p.chosen = (int)p.candidates.size() - 1;
+}
 
 // Finds or makes the plan of a product.  Called with g_mu held.
 int plan_for(const Key& key, size_t workspace_bytes, Plan** out) {
@@ -86,6 +116,7 @@ int plan_for(const Key& key, size_t workspace_bytes, Plan** out) {
         if (p.desc) hipblasLtMatmulDescDestroy(p.desc);
         return ok ? IC_ERR_NO_ALGORITHM : IC_ERR_LIBRARY;
     }
+    borrow_from_neighbour(key, p, workspace_bytes);
     *out = &g_plans.emplace(key, std::move(p)).first->second;
     return IC_OK;
 }
@@ -125,7 +156,8 @@ IC_EXPORT int ic_matmul(const void* A, int a_dtype, const void* W, void* C, int 
 
 // Times every algorithm the library proposes for this product (reps launches each, after one to warm up) on
 // `stream` and keeps the fastest, if it beats the library's first choice by 3 %, for later ic_matmul calls of the
-// same shape.  Synchronises the stream.
+// same shape, and of shapes first seen later that differ only by a row count within an eighth of this one.
+// Synchronises the stream.
 // flush (may be nullptr): device memory, larger than the chip's caches, that is overwritten before every timed
 // launch, so that the operands come from memory as a model's weights do and not from the last launch's cache lines.
 // Returns the number of algorithms tried (>= 1) or an error code (< 0).
@@ -198,5 +230,6 @@ IC_EXPORT int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C,
     if (tried == 0) return IC_ERR_LIBRARY;
     // the library's own first choice stays unless another is clearly (3 %) faster: timing noise must not pick
     p->chosen = (first > 0.f && best > 0.97f * first) ? 0 : best_i;
+    p->timed = true;
     return tried;
 }

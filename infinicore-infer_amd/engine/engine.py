@@ -334,9 +334,9 @@ class Engine:
         fastest algorithm: one dummy step per count is run in which every library product first times
         the algorithms the library has for its shape on the device and keeps the best.  Between
         timed launches 512 MB of scratch memory are overwritten: in a model every product's weights
-        come from memory, not from the cache lines a repeated launch would find.  Other
-        shapes keep the library's first choice and cost nothing.  Optional; results live for this
-        process."""
+        come from memory, not from the cache lines a repeated launch would find.  A step whose
+        token count is within an eighth of a timed one takes that one's algorithms; other shapes keep
+        the library's first choice and cost nothing.  Optional; results live for this process."""
         from ..parts import linear as _linear
         _linear.TUNE_LIBRARY = True
         _linear.TUNE_FLUSH = torch.empty(512 << 20, dtype=torch.uint8, device=self.device)
