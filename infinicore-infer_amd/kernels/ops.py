@@ -351,24 +351,49 @@ class NoLibraryAlgorithm(KernelError):
     """The library proposes no algorithm for a product."""
 
 
+_matmul_types = {}      # (operand dtype, result dtype) -> (codes) or None: asked of the library once
+
+
 def _matmul_args(a, w, out, what):
-    _dev(a, w, out)
+    """Checks a product's operands and returns (M, N, K, operand code, result code, row strides of a, w, out).
+    Written for few attribute lookups: this runs four times a layer."""
+    if not (a.is_cuda and w.is_cuda and out.is_cuda):
+        _dev(a, w, out)
     M, K = a.shape
-    N = w.shape[0]
-    _need(w.shape[1] == K and tuple(out.shape) == (M, N), what + ": shape mismatch")
-    _need(a.dtype == w.dtype and a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, what + ": layout")
-    _need(bool(get_lib().ic_matmul_supported(dtype_code(a.dtype), dtype_code(out.dtype))), what + ": unsupported types")
-    return M, N, K
+    N, Kw = w.shape
+    Mo, No = out.shape
+    sa, sa1 = a.stride()
+    sw, sw1 = w.stride()
+    so, so1 = out.stride()
+    if Kw != K or Mo != M or No != N:
+        raise KernelError(what + ": shape mismatch")
+    if sa1 != 1 or sw1 != 1 or so1 != 1:
+        raise KernelError(what + ": layout")
+    key = (a.dtype, w.dtype, out.dtype)
+    codes = _matmul_types.get(key, False)
+    if codes is False:
+        codes = None
+        if a.dtype == w.dtype and a.dtype in _DT and out.dtype in _DT and \
+                get_lib().ic_matmul_supported(_DT[a.dtype], _DT[out.dtype]):
+            codes = (_DT[a.dtype], _DT[out.dtype])
+        _matmul_types[key] = codes
+    if codes is None:
+        raise KernelError(what + ": unsupported types")
+    return M, N, K, codes[0], codes[1], sa, sw, so
 
 
 def matmul_library(a, w, out, alpha: float = 1.0):
     """out[M, N] = alpha * a[M, K] @ w[N, K]^T through the library (hipBLASLt), any number of rows.
     bfloat16 operands with a bfloat16 or float32 result, or all float32."""
-    M, N, K = _matmul_args(a, w, out, "matmul_library")
-    ws = _workspace(a.device)
-    st = get_lib().ic_matmul(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), out.data_ptr(), dtype_code(out.dtype),
-                             M, N, K, a.stride(0), w.stride(0), out.stride(0), float(alpha), ws.data_ptr(), ws.numel(),
-                             _stream())
+    M, N, K, ca, cc, sa, sw, so = _matmul_args(a, w, out, "matmul_library")
+    stream = _stream()
+    ws = _matmul_workspace.get((a.device, stream))
+    if ws is None:
+        ws = _workspace(a.device)
+    st = get_lib().ic_matmul(a.data_ptr(), ca, w.data_ptr(), out.data_ptr(), cc, M, N, K, sa, sw, so, alpha,
+                        ws.data_ptr(), MATMUL_WORKSPACE_BYTES, stream)
+    if st == 0:
+        return out
     if st == -4:
         raise NoLibraryAlgorithm("matmul_library: no algorithm for %d x %d x %d" % (M, N, K))
     if st == -3:
@@ -381,13 +406,13 @@ def matmul_library_tune(a, w, out, reps: int = 5, flush=None) -> int:
     """Times the library's algorithms for this product's shape and keeps the fastest; returns how many it tried.
     flush: a device tensor larger than the chip's caches; it is overwritten before every timed launch, so that the
     algorithms are compared with operands that come from memory, as a model's weights do."""
-    M, N, K = _matmul_args(a, w, out, "matmul_library_tune")
+    M, N, K, ca, cc, sa, sw, so = _matmul_args(a, w, out, "matmul_library_tune")
     ws = _workspace(a.device)
     if flush is not None:
         _dev(a, flush)
         _need(flush.is_contiguous(), "matmul_library_tune: flush must be contiguous")
-    n = get_lib().ic_matmul_tune(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), out.data_ptr(), dtype_code(out.dtype),
-                                 M, N, K, a.stride(0), w.stride(0), out.stride(0), ws.data_ptr(), ws.numel(),
+    n = get_lib().ic_matmul_tune(a.data_ptr(), ca, w.data_ptr(), out.data_ptr(), cc, M, N, K, sa, sw, so,
+                                 ws.data_ptr(), ws.numel(),
                                  flush.data_ptr() if flush is not None else None,
                                  flush.numel() * flush.element_size() if flush is not None else 0, int(reps), _stream())
     if n < 0:
