@@ -386,7 +386,7 @@ def test_library_float32_product_is_true_float32():
 
 
 # ---------------------------------------------------------------------------
-@pytest.mark.parametrize("V", [256, 509, 122753])
+@pytest.mark.parametrize("V", [256, 509, 122753, 300001])     # the last: beyond what the per-run masses cover
 def test_sampling(V):
     ops = _ops()
     g = torch.Generator().manual_seed(18)
