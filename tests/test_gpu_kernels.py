@@ -417,6 +417,47 @@ def test_sampling(V):
     assert out.cpu().tolist() == want
 
 
+@pytest.mark.parametrize("V", [5003, 122753])
+def test_sampling_where_the_short_list_does_not_apply_or_ties_cross_its_edge(V):
+    """Rows made so that the kernel's ways through a row all occur: ties across the k-th place (kept
+    together), a k so large and a distribution so flat that the candidates do not fit in LDS, all logits
+    equal, all negative, a draw at either end."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(23)
+    rows, params = [], []
+
+    def add(row, t, k, p, u):
+        rows.append(row)
+        params.append((t, k, p, u))
+
+    base = torch.randn(V, generator=g) * 3
+    tied = base.clone()
+    top = torch.topk(tied, 12).indices
+    tied[top[4:]] = float(tied[top[4]])                         # places 5..12 share one value
+    for k in (5, 6, 12, 13):
+        add(tied, 1.0, k, 1.0, 0.999)
+        add(tied, 0.8, k, 0.7, 0.5)
+    add(base, 1.0, V - 1, 1.0, 0.37)                            # top-k cuts one token: no short list
+    add(base, 1.5, V // 3, 0.9, 0.61)
+    add(base * 0.01, 1.0, 0, 0.9, 0.42)                         # nearly flat: top-p keeps most of the row
+    add(torch.full((V,), 1.25), 1.0, 7, 0.5, 0.73)              # all equal: everything stays together
+    add(-10.0 - torch.rand(V, generator=g), 0.9, 40, 0.8, 0.2)  # all negative
+    add(base, 1.0, 50, 0.9, 0.0)                                # the draw's ends
+    add(base, 1.0, 50, 0.9, 1.0)
+    add(base, 1.0, 0, 1.0, 0.0)
+    add(base, 1.0, 0, 1.0, 1.0)
+    add(base, 0.05, 0, 0.999, 0.5)                              # a cold temperature: most masses round to zero
+    logits = torch.stack(rows)
+    R = len(rows)
+    col = lambda j, dt: torch.tensor([q[j] for q in params], dtype=dt).to(DEV)
+    out = torch.empty(R, dtype=torch.int32, device=DEV)
+    ops.sample(logits.to(DEV), out, col(0, torch.float32), col(1, torch.int32), col(2, torch.float32), col(3, torch.float32))
+    got = out.cpu().tolist()
+    for r, (t, k, p, u) in enumerate(params):
+        want = P.plain_sample(logits[r], t, k, p, float(torch.tensor(u, dtype=torch.float32)))
+        assert got[r] == want, "row %d (T=%g k=%d p=%g u=%g): got %d, plain %d" % (r, t, k, p, u, got[r], want)
+
+
 def test_sampling_distribution():
     """Many draws at temperature 1 follow softmax (chi-square against torch.softmax)."""
     ops = _ops()
