@@ -353,6 +353,7 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
     if (hi > pos + 1) hi = pos + 1;
 
     const int lane = threadIdx.x & 63, wave = threadIdx.x >> 6;
+    const float scale2 = scale * 1.4426950408889634f;   // scores and running maxima in units of log 2: exp2 is one instruction
     const int lr = lane & 15, lg = lane >> 4;      // row / column of a tile, and the lane group
     const size_t head_stride = (size_t)page_size * DH;
     const size_t page_stride = (size_t)nkvh * head_stride;
@@ -452,18 +453,18 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
 #pragma unroll
                 for (int e = 0; e < 4; ++e) {
                     const int key = kt + 16 * s2 + 4 * lg + e;
-                    const float x = (key < hi) ? sacc[s2][e] * scale : -INFINITY;
+                    const float x = (key < hi) ? sacc[s2][e] * scale2 : -INFINITY;     // in units of log 2
                     sv[4 * s2 + e] = x;
                     mloc = fmaxf(mloc, x);
                 }
             mloc = fmaxf(mloc, __shfl_xor(mloc, 16, kWave));
             mloc = fmaxf(mloc, __shfl_xor(mloc, 32, kWave));
             const float m_new = fmaxf(m, mloc);     // finite: every tile has at least one key
-            const float corr = expf(m - m_new);
+            const float corr = __builtin_amdgcn_exp2f(m - m_new);
             float rs = 0.f;
             gq_v8f pf;
 #pragma unroll
-            for (int e = 0; e < 8; ++e) { const float p = expf(sv[e] - m_new); pf[e] = p; rs += p; }
+            for (int e = 0; e < 8; ++e) { const float p = __builtin_amdgcn_exp2f(sv[e] - m_new); pf[e] = p; rs += p; }
             rs += __shfl_xor(rs, 16, kWave);
             rs += __shfl_xor(rs, 32, kWave);
             l = l * corr + rs;
@@ -503,7 +504,7 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
             float a = 0.f, ll = 0.f;
             if (mm != -INFINITY) {
                 for (int w = 0; w < kDecWaves; ++w) {
-                    const float cw = expf(sm_ml[w][j][0] - mm);
+                    const float cw = __builtin_amdgcn_exp2f(sm_ml[w][j][0] - mm);
                     a += sm_o[(w * 16 + j) * DH + d] * cw;
                     ll += sm_ml[w][j][1] * cw;
                 }
@@ -515,7 +516,7 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
             }
             const size_t pidx = ((size_t)n * nh + h) * nsplit + split;
             part_acc[pidx * DH + d] = a;
-            if (d == 0) { part_ml[pidx * 2] = mm; part_ml[pidx * 2 + 1] = ll; }
+            if (d == 0) { part_ml[pidx * 2] = mm * 0.6931471805599453f; part_ml[pidx * 2 + 1] = ll; }   // natural units for the second pass
         }
         __syncthreads();                            // sm_o (the V tiles) is reused by the next chunk
     }

@@ -41,6 +41,12 @@ __device__ __forceinline__ uint16_t f32_to_bf16_bits(float f) {
 }
 
 // ---- reductions over a 64-lane wave ------------------------------------------
+// up * silu(gate) with the hardware's exp2 and reciprocal (each good to an ulp): for results that are
+// rounded to bfloat16.  The float32 path divides and calls expf.
+__device__ __forceinline__ float silu_mul_fast(float g, float u) {
+    return u * g * __builtin_amdgcn_rcpf(1.0f + __builtin_amdgcn_exp2f(-1.4426950408889634f * g));
+}
+
 __device__ __forceinline__ float wave_sum(float v) {
 #pragma unroll
     for (int o = 32; o > 0; o >>= 1) v += __shfl_xor(v, o, kWave);

@@ -256,7 +256,7 @@ __global__ void swiglu_vec8_kernel(const bf16* __restrict__ gu, bf16* __restrict
         load4(gp, g); load4(gp + 4, g + 4);
         load4(gp + di, u); load4(gp + di + 4, u + 4);
 #pragma unroll
-        for (int e = 0; e < 8; ++e) o[e] = u[e] * (g[e] / (1.0f + expf(-g[e])));
+        for (int e = 0; e < 8; ++e) o[e] = silu_mul_fast(g[e], u[e]);
         bf16* op = out + t * (size_t)di + j;
         store4(op, o); store4(op + 4, o + 4);
     }

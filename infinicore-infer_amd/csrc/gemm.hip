@@ -278,7 +278,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
                     g = to_f32(from_f32<TC>(alpha * g));
                     u = to_f32(from_f32<TC>(alpha * u));
                     const int n = n0 + 16 * gi + 4 * kq + e;
-                    if (m < M && n < sw_end) C[(size_t)m * ldc + n] = from_f32<TC>(u * (g / (1.0f + expf(-g))));
+                    if (m < M && n < sw_end) C[(size_t)m * ldc + n] = from_f32<TC>(silu_mul_fast(g, u));
                 }
         }
         return;
