@@ -44,7 +44,8 @@ def test_embed(dtype, T, d, V):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("T,d,eps", [(1, 64, 1e-5), (33, 200, 1e-6), (17, 2304, 1e-5), (5, 4097, 1e-2)])
+@pytest.mark.parametrize("T,d,eps", [(1, 64, 1e-5), (33, 200, 1e-6), (17, 2304, 1e-5), (5, 4097, 1e-2),
+                                     (2051, 200, 1e-5), (1027, 5000, 1e-5)])     # many rows
 def test_rmsnorm(dtype, T, d, eps):
     g = torch.Generator().manual_seed(2)
     x = torch.randn(T, d, generator=g) * 3
@@ -64,7 +65,7 @@ def test_rmsnorm(dtype, T, d, eps):
 
 
 @pytest.mark.parametrize("dtype", DT)
-@pytest.mark.parametrize("T,d", [(3, 96), (40, 200), (9, 2304)])
+@pytest.mark.parametrize("T,d", [(3, 96), (40, 200), (9, 2304), (2050, 200), (1100, 2304), (1030, 5000)])   # the last three: many rows
 def test_add_rmsnorm_and_residual_add(dtype, T, d):
     g = torch.Generator().manual_seed(3)
     x = torch.randn(T, d, generator=g)
