@@ -216,14 +216,19 @@ class Engine:
             row0 = req_start[r]
             want_rows.extend(row0 + int(w) for w in e.want)
             if n == 1:
-                decode_rows.append(row0)
+                decode_rows.append((p0, row0))
                 max_ctx = max(max_ctx, p0 + 1)
             else:
                 for o in range(0, n, self._tile_rows):
                     tiles.append((r, row0 + o, min(self._tile_rows, n - o), p0 + o))
         state_slots = [self.cache.state_slot(e.req_id) for e in entries]
-        # tiles that see the most keys go first, so the longest blocks do not form the tail
+        # tiles that see the most keys go first, so the longest blocks do not form the tail; likewise the
+        # single tokens (their order is free: each names its row), unless all rows are single tokens and
+        # the kernel takes the rows as they lie
         tiles.sort(key=lambda t: -(t[3] + t[2]))
+        if len(decode_rows) < T:
+            decode_rows.sort(key=lambda pr: -pr[0])
+        decode_rows = [row for _, row in decode_rows]
 
         n_groups = len(self.groups)
         tables = [[self.cache.block_table(e.req_id, g) for e in entries] for g in range(n_groups)]
