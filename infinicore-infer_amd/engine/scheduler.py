@@ -34,7 +34,7 @@ from .engine import StepEntry
 from .tasks import InferTask
 
 
-@dataclass
+@dataclass(eq=False)               # compared by identity: membership tests must not compare token lists
 class _Running:
     task: InferTask
     feed: List[int]                  # tokens of this request still to be computed (prompt, or prompt + generated)
