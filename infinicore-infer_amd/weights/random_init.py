@@ -85,3 +85,23 @@ def write_random_model(folder: str, config: dict, seed: int, std: float = 0.02, 
         json.dump(cfg, f, indent=1)
     save_file(sd, os.path.join(folder, "model.safetensors"), metadata={"format": "pt", "seed": str(seed)})
     return folder
+
+
+def main(argv=None) -> int:
+    """python -m infinicore_infer_amd.weights --config config.json --seed S --out DIR
+    writes a model folder (config.json, model.safetensors) with random weights for that configuration."""
+    import argparse
+    ap = argparse.ArgumentParser(prog="python -m infinicore_infer_amd.weights", description="write a model folder with random weights")
+    ap.add_argument("--config", required=True, help="a config.json of the architecture")
+    ap.add_argument("--out", required=True, help="folder to write (created if missing)")
+    ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--std", type=float, default=0.02, help="standard deviation of matrices and embeddings")
+    ap.add_argument("--norm-std", type=float, default=0.0, help="norm weights are 1 + N(0, this)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"])
+    args = ap.parse_args(argv)
+    with open(args.config, encoding="utf-8") as f:
+        config = json.load(f)
+    folder = write_random_model(args.out, config, args.seed, args.std, args.norm_std,
+                                {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype])
+    print("wrote %s" % folder)
+    return 0

@@ -102,3 +102,21 @@ def test_untied_head_only_backs_the_embedding(tmp_path):
     m = _model("A")
     m.load_from_dir(folder)
     assert m.head.weight is m.embedding.table
+
+
+def test_random_weights_from_the_command_line(tmp_path):
+    """python -m infinicore_infer_amd.weights --config .. --seed .. --out ..: the folder it writes equals
+    the one the function writes for the same configuration and seed."""
+    import subprocess
+    import sys
+    cfg_file = tmp_path / "cfg.json"
+    cfg_file.write_text(json.dumps(H.TINY_B))
+    root = os.path.dirname(os.path.dirname(os.path.abspath(__file__)))
+    out = tmp_path / "by_cli"
+    r = subprocess.run([sys.executable, "-m", "infinicore_infer_amd.weights", "--config", str(cfg_file), "--seed", "5",
+                        "--std", "0.05", "--norm-std", "0.1", "--out", str(out)], cwd=root, capture_output=True, text=True)
+    assert r.returncode == 0, r.stderr
+    ref = write_random_model(str(tmp_path / "by_call"), H.TINY_B, 5, std=0.05, norm_std=0.1)
+    a, b = load_file(str(out / "model.safetensors")), load_file(os.path.join(ref, "model.safetensors"))
+    assert sorted(a) == sorted(b) and all(torch.equal(a[k], b[k]) for k in a)
+    assert json.load(open(out / "config.json"))["vocab_size"] == H.TINY_B["vocab_size"]
