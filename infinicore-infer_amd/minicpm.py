@@ -175,7 +175,7 @@ class MiniCPMForCausalLM:
 
 USAGE = ("Usage: python -m infinicore_infer_amd.minicpm [--amd] <path/to/model_dir> [n_device] "
          "[--dtype bfloat16|float32] [--max-tokens N] [--prompt TEXT | --prompt-ids 1,2,3] [--max-steps N] "
-         "[--temperature T] [--topk K] [--topp P] [--seed S]")
+         "[--temperature T] [--topk K] [--topp P] [--seed S] [--page-size 16|32|64] [--cache-tokens N]")
 
 
 def test(argv=None):
@@ -205,8 +205,11 @@ def test(argv=None):
     ap.add_argument("--topk", type=int, default=1)
     ap.add_argument("--topp", type=float, default=1.0)
     ap.add_argument("--seed", type=int, default=0)
+    ap.add_argument("--page-size", type=int, default=64, choices=(16, 32, 64), help="tokens per cache page")
+    ap.add_argument("--cache-tokens", type=int, default=None, help="tokens the page pool holds (default: four contexts)")
     args = ap.parse_args(argv)
-    model = MiniCPMForCausalLM(model_path, "cuda:0", ndev, max_tokens=args.max_tokens, dtype=_DTYPES[args.dtype])
+    model = MiniCPMForCausalLM(model_path, "cuda:0", ndev, max_tokens=args.max_tokens, dtype=_DTYPES[args.dtype],
+                               cache_tokens=args.cache_tokens, page_size=args.page_size)
     prompt = [int(t) for t in args.prompt_ids.split(",")] if args.prompt_ids else args.prompt
     model.generate(prompt, args.max_steps, topp_=args.topp, topk_=args.topk, temperature_=args.temperature,
                    seed=args.seed)
