@@ -147,6 +147,10 @@ class MiniCPMConfig:
             raise ConfigError("dim_model_base must be positive")
         if self.logit_scale_rule not in ("reference", "mup"):
             raise ConfigError("logit_scale_rule must be 'reference' or 'mup'")
+        if self.mup and self.logit_scale_rule == "reference" and self.hidden_size // self.dim_model_base == 0:
+            raise ConfigError("dim_model_base (%d) above hidden_size (%d): the integer ratio that scales the "
+                              "logits (hidden_size // dim_model_base) is 0 and every logit would be 0"
+                              % (self.dim_model_base, self.hidden_size))
         rs = self.rope_scaling
         if rs is not None:
             half = self.head_dim // 2

@@ -58,6 +58,9 @@ def test_missing_and_bad_keys_are_named():
         config_from_dict(dict(H.TINY_C, rope_scaling=dict(H.TINY_C["rope_scaling"], short_factor=[1.0] * 3)))
     with pytest.raises(ConfigError):
         config_from_dict(dict(H.TINY_C, rope_scaling={"type": "yarn"}))
+    with pytest.raises(ConfigError) as e:      # the reference's integer width ratio would be 0: all logits 0
+        config_from_dict(dict(H.TINY_A, dim_model_base=H.TINY_A["hidden_size"] + 1))
+    assert "dim_model_base" in str(e.value)
 
 
 def test_registry_lookup_and_unknown_architecture():
