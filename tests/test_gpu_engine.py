@@ -227,6 +227,52 @@ def test_recorded_steps_with_library_products_equal_eager_ones(tmp_path_factory,
     assert a.graph_replays == 10 and b.graph_replays == 0
 
 
+def _random_configuration(seed):
+    """A tiny configuration drawn from the seed: head sizes in steps of 16, any number of kv heads and of
+    query heads on each, widths and inner sizes that are multiples of 8, of 4, of 2, or odd."""
+    import random
+    rng = random.Random(seed)
+    dh = rng.choice([16, 32, 48, 64, 80, 96, 112, 128])
+    nkvh = rng.choice([1, 2, 3, 5])
+    nh = nkvh * rng.choice([1, 1, 2, 3, 4, 7])
+    d = rng.choice([nh * dh, 8 * rng.randint(5, 40), 4 * rng.randint(11, 60), 2 * rng.randint(21, 99), rng.randint(40, 300)])
+    di = rng.choice([8 * rng.randint(6, 50), 4 * rng.randint(13, 90), rng.randint(50, 400)])
+    max_pos = rng.choice([64, 128, 200, 320])
+    cfg = dict(model_type=rng.choice(["minicpm", "fm9g"]), vocab_size=rng.randint(50, 700), hidden_size=d,
+               num_hidden_layers=rng.randint(1, 3), num_attention_heads=nh, num_key_value_heads=nkvh, head_dim=dh,
+               intermediate_size=di, max_position_embeddings=max_pos, rms_norm_eps=rng.choice([1e-5, 1e-6, 1e-3]),
+               rope_theta=rng.choice([1e4, 1e6, 5e4]), scale_emb=rng.choice([1.0, 12, 4.0]),
+               dim_model_base=rng.choice([d, max(1, d // 4)]), scale_depth=rng.choice([1.0, 1.4, 2.0]),
+               tie_word_embeddings=rng.random() < 0.5, eos_token_id=2)
+    if rng.random() < 0.3:
+        cfg["rope_scaling"] = dict(type="longrope", original_max_position_embeddings=max_pos // 2,
+                                   short_factor=[1.0 + 0.05 * i for i in range(dh // 2)],
+                                   long_factor=[1.0 + 0.09 * i for i in range(dh // 2)])
+    lens = [min(max_pos, n) for n in (rng.randint(1, max_pos), rng.randint(1, 40), 65, 17)]
+    return cfg, lens, rng.choice([16, 64])
+
+
+@pytest.mark.parametrize("seed", [3, 11, 29, 176, 251, 301, 412, 733])
+def test_random_configurations(tmp_path_factory, seed):
+    """Configurations nobody chose: each request's last tokens one by one and a mixed trace, in both
+    dtypes, against the plain implementation."""
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.weights import write_random_model
+    import os
+    cfg, lens, page = _random_configuration(seed)
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "model_random_%d" % seed)
+    write_random_model(folder, cfg, seed=seed, std=min(0.05, cfg["hidden_size"] ** -0.5), norm_std=0.1)
+    sd = H.load_state_dict(folder)
+    requests = {"r%d" % i: H.random_tokens(cfg["vocab_size"], n, seed * 13 + i) for i, n in enumerate(lens)}
+    for dname, dtype, tol in DTYPES:
+        ref = H.plain_logits(cfg, sd, requests, dtype == torch.bfloat16)
+        for maker in (H.trace_last_one_by_one, H.trace_mixed):
+            steps, max_tokens = maker(requests)
+            engine = Engine.from_dir(folder, dtype=dtype, max_tokens=max(max_tokens, 64), page_size=page, max_requests=8)
+            H.compare(H.run_trace(engine, steps), ref, tol, "seed %d %s %s %r" % (seed, dname, maker.__name__, cfg))
+            engine.cache.check_invariants()
+
+
 def test_trace_run_program(tmp_path):
     """bin/trace_run as a program: files, 'done' lines, exit status, and the logits themselves."""
     import json, os, subprocess, sys
