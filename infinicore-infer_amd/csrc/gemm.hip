@@ -6,7 +6,7 @@
 // NT tiles of 16 weight rows and a share of K (k-steps of 32, dealt in turn; WPB is 4, 8
 // or 16 so that narrow matrices still fill the chip); lane
 // (r = l%16, kq = l/16) loads 16 bytes W[n0+r][k0+8kq..+7] and the matching
-// 16 bytes of each A row tile, and feeds them to two v_mfma_f32_16x16x16_bf16
+// 16 bytes of each A row tile, and feeds them to one v_mfma_f32_16x16x32_bf16
 // as A and B operands.  Both operands use the same lane->k mapping, so the
 // order of k inside a step does not matter.  The waves' partial sums meet in LDS.
 // Two variants of the walk over K: OWN_K gives each wave one contiguous run of
@@ -14,7 +14,7 @@
 // k-steps when at most 16 / AG rows are in use (the spare lanes carry the other
 // steps' data and a row rotation hands it over).
 //
-// 16x16x16 layout (lane l): A[i = l%16][k = 4(l/16)..+3], B[k = 4(l/16)..+3][j = l%16],
+// 16x16x32 layout (lane l): A[i = l%16][k = 8(l/16)..+7], B[k = 8(l/16)..+7][j = l%16],
 // D[i = 4(l/16) + e][j = l%16], e = 0..3.
 #include "common.h"
 #include <utility>
@@ -233,8 +233,13 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
             for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(wlo[u][nt], alo[u][mt], acc[nt][mt], 0, 0, 0);
-                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x16bf16_1k(whi[u][nt], ahi[u][mt], acc[nt][mt], 0, 0, 0);
+                    // one 16x16x32 product per k-step: a lane's 8 elements of W and of A are k = 8 kq .. 8 kq + 7 of the step
+                    typedef short v8s __attribute__((ext_vector_type(8)));
+                    typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+                    const v8s w8 = __builtin_shufflevector(wlo[u][nt], whi[u][nt], 0, 1, 2, 3, 4, 5, 6, 7);
+                    const v8s a8 = __builtin_shufflevector(alo[u][mt], ahi[u][mt], 0, 1, 2, 3, 4, 5, 6, 7);
+                    acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w8), __builtin_bit_cast(v8b, a8),
+                                                                          acc[nt][mt], 0, 0, 0);
                 }
     }
     if (wave > 0) {
