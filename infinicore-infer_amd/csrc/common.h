@@ -15,6 +15,7 @@
 #define IC_OK 0
 #define IC_ERR_ARG (-1)
 #define IC_ERR_UNSUPPORTED (-2)
+#define IC_ERR_TOO_LARGE (-5)     // beyond the fixed capacity of an entry point that allocates nothing
 
 // dtype codes shared with the Python binding.
 #define IC_F32 0

@@ -2,7 +2,8 @@
 //
 // Every function launches on `stream` and returns 0 when the launch was queued,
 // IC_ERR_ARG (-1) for a shape, stride, alignment or size the kernel does not take,
-// IC_ERR_UNSUPPORTED (-2) for a dtype or head size without a kernel, or the
+// IC_ERR_UNSUPPORTED (-2) for a dtype or head size without a kernel, IC_ERR_TOO_LARGE (-5)
+// for a size beyond the fixed capacity of an entry point that allocates nothing, or the
 // (positive) hipError_t of a failed launch.  Nothing here allocates device memory;
 // scratch buffers are passed in by the caller.  dtype codes: 0 = float32, 1 = bfloat16.
 //
@@ -91,6 +92,15 @@ int ic_matmul_tune(const void* A, int a_dtype, const void* W, void* C, int c_dty
 // ---- sampling.hip -----------------------------------------------------------------------------------
 // Greedy choice per row; scratch_val / scratch_idx: 64 * n_rows elements.
 int ic_argmax(const float* logits, long long row_stride, int n_rows, int V, float* scratch_val, int* scratch_idx, int* out, hipStream_t stream);
+// For callers that cannot allocate device memory (code under HIP graph capture, tight serving loops,
+// harnesses that forbid it); it has no counterpart in the reference.  The same result as ic_argmax, with the
+// partial results in the library's own static device memory (512 KB on every GPU the library runs on, held
+// until the process ends) instead of a scratch buffer from the caller: nothing is allocated or freed, here
+// or in anything it calls.  At most ic_argmax_static_max_rows() (1024) rows: more returns IC_ERR_TOO_LARGE
+// (-5) and launches nothing.  The device of `stream` must be the current device.  All calls on one GPU share
+// that memory: calls that overlap on one GPU (two streams, two threads) race; calls in stream order do not.
+int ic_argmax_static_max_rows();
+int ic_argmax_static(const float* logits, long long row_stride, int n_rows, int V, int* out, hipStream_t stream);
 // Temperature / top-k / top-p with one uniform draw per row; temperature == nullptr: argmax.
 int ic_sample(const float* logits, long long row_stride, int n_rows, int V, const float* temperature, const int* top_k, const float* top_p, const float* uniform, int* out, hipStream_t stream);
 

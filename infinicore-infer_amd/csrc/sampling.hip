@@ -25,6 +25,8 @@
 //   top_p * total (equal values stay together); the token is the first, in
 //   vocabulary order, whose cumulated kept mass reaches u * kept_total.
 #include "common.h"
+#include <atomic>
+#include <mutex>
 
 constexpr int kSampleThreads = 1024;
 constexpr int kSampleWaves = kSampleThreads / 64;
@@ -483,6 +485,62 @@ IC_EXPORT int ic_argmax(const float* logits, long long row_stride, int n_rows, i
     int st = ic_launch_status();
     if (st) return st;
     hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(64), 0, stream, scratch_val, scratch_idx, out);
+    return ic_launch_status();
+}
+
+// ---- greedy choice for callers that cannot allocate ------------------------------------------
+// The partial results of the two-stage argmax live in a file-scope device array instead of a
+// buffer the caller brings: kArgmaxStaticRows rows x 64 chunks x (float value, int index) = 512 KB,
+// held by every GPU the library runs on until the process ends.  In host code the array's name is
+// only a stand-in; its device address is asked for once per device and kept.
+constexpr int kArgmaxStaticRows = 1024;
+constexpr int kMaxDevices = 64;
+static __device__ __align__(256) unsigned char scratch[(size_t)kArgmaxStaticRows * kArgmaxChunks * (sizeof(float) + sizeof(int))];
+static std::atomic<void*> g_scratch_ptr[kMaxDevices];
+static std::mutex g_scratch_mutex;
+
+// Device address of `scratch` on the current device (asked for at the first call on that device).
+static int static_scratch(void** ptr) {
+    int dev = -1;
+    hipError_t e = hipGetDevice(&dev);
+    if (e != hipSuccess) return (int)e;
+    if (dev < 0 || dev >= kMaxDevices) return IC_ERR_ARG;
+    void* p = g_scratch_ptr[dev].load(std::memory_order_acquire);
+    if (!p) {
+        std::lock_guard<std::mutex> hold(g_scratch_mutex);
+        p = g_scratch_ptr[dev].load(std::memory_order_relaxed);
+        if (!p) {
+            e = hipGetSymbolAddress(&p, HIP_SYMBOL(scratch));
+            if (e != hipSuccess) return (int)e;
+            if (!p) return (int)hipErrorInvalidSymbol;
+            g_scratch_ptr[dev].store(p, std::memory_order_release);
+        }
+    }
+    *ptr = p;
+    return IC_OK;
+}
+
+IC_EXPORT int ic_argmax_static_max_rows() { return kArgmaxStaticRows; }
+
+// ic_argmax with the library's own scratch memory: no allocation, here or in anything it calls.
+// Every (row, chunk) cell the second stage reads is written by the first stage of the same call, so
+// nothing has to be cleared between calls; calls that overlap on one GPU share the array and race.
+IC_EXPORT int ic_argmax_static(const float* logits, long long row_stride, int n_rows, int V, int* out,
+                               hipStream_t stream) {
+    if (n_rows <= 0) return IC_OK;
+    if (n_rows > kArgmaxStaticRows) return IC_ERR_TOO_LARGE;
+    if (V <= 0 || row_stride < V || !logits || !out) return IC_ERR_ARG;
+    void* base = nullptr;
+    int st = static_scratch(&base);
+    if (st) return st;
+    float* pval = reinterpret_cast<float*>(base);
+    int* pidx = reinterpret_cast<int*>(reinterpret_cast<unsigned char*>(base)
+                                       + (size_t)kArgmaxStaticRows * kArgmaxChunks * sizeof(float));
+    hipLaunchKernelGGL(argmax_partial_kernel, dim3(kArgmaxChunks, n_rows), dim3(256), 0, stream, logits,
+                       row_stride, V, pval, pidx);
+    st = ic_launch_status();
+    if (st) return st;
+    hipLaunchKernelGGL(argmax_final_kernel, dim3(n_rows), dim3(64), 0, stream, pval, pidx, out);
     return ic_launch_status();
 }
 

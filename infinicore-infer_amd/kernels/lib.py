@@ -56,6 +56,8 @@ _SIGNATURES = {
     "ic_attn_prefill_groups": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
+    "ic_argmax_static_max_rows": [],
+    "ic_argmax_static": [_P, _LL, _I, _I, _P, _P],
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],
     "ic_gemm_nt_residual_parts": [_I],
     "ic_gemm_nt_supported": [_I, _I, _I],
@@ -102,4 +104,6 @@ def check(status: int, what: str) -> None:
         raise KernelError("%s: bad argument (shape, stride, alignment or size outside what the kernel takes)" % what)
     if status == -2:
         raise KernelError("%s: unsupported dtype or head size" % what)
+    if status == -5:
+        raise KernelError("%s: more rows than the entry point's fixed scratch memory holds" % what)
     raise KernelError("%s: HIP error %d at launch" % (what, status))

@@ -269,6 +269,19 @@ def argmax(logits, out, scratch_val, scratch_idx):
     return out
 
 
+def argmax_static(logits, out):
+    """argmax with the library's own static scratch memory: allocates nothing, takes at most
+    ``get_lib().ic_argmax_static_max_rows()`` rows; calls that overlap on one GPU race."""
+    _dev(logits, out)
+    R, V = logits.shape
+    _need(logits.dtype == torch.float32 and logits.stride(1) == 1, "argmax_static: logits must be float32 rows")
+    _i32(out, "out")
+    _need(out.numel() >= R, "argmax_static: out too short")
+    check(get_lib().ic_argmax_static(logits.data_ptr(), logits.stride(0), R, V, out.data_ptr(), _stream()),
+          "argmax_static")
+    return out
+
+
 def gemm_nt_supported(a_dtype, w_dtype, c_dtype) -> bool:
     try:
         return bool(get_lib().ic_gemm_nt_supported(dtype_code(a_dtype), dtype_code(w_dtype), dtype_code(c_dtype)))
