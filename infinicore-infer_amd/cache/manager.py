@@ -165,6 +165,21 @@ class CacheManager:
         e.length += n_new
         return start
 
+    def truncate(self, req_id, length: int) -> None:
+        """Undo appends: the request holds ``length`` tokens again and the pages beyond them are
+        given back.  Only for a step that failed before it ran (no window page of it was trimmed)."""
+        e = self.requests[req_id]
+        if length > e.length or length < 0:
+            raise CacheError("truncate: request %r holds %d tokens, %d asked" % (req_id, e.length, length))
+        keep = self._pages_for(length)
+        for g, table in enumerate(e.tables):
+            while len(table) > keep:
+                p = table.pop()
+                if p >= 0:
+                    self.pools[g].free(p)
+            e.first_live[g] = min(e.first_live[g], len(table))
+        e.length = length
+
     def trim(self, req_id) -> int:
         """Give back the pages of window groups that no later token can read.
         Call after the step that appended has been launched.  Returns the count."""

@@ -64,6 +64,10 @@ class MiniCPMConfig:
     # "reference": the final hidden state is multiplied by hidden_size // dim_model_base,
     # as scripts/jiuge.py:108,199 does.  "mup": divided by hidden_size / dim_model_base.
     logit_scale_rule: str = "reference"
+    # The serving cap on a request's length (the reference's max_tokens argument,
+    # scripts/jiuge.py:128-130).  It bounds positions, the rotary tables and the cache; the
+    # checkpoint's own max_position_embeddings stays what long-context scaling is derived from.
+    context_cap: Optional[int] = None
 
     # ---- reading ---------------------------------------------------------
     @classmethod
@@ -109,8 +113,8 @@ class MiniCPMConfig:
             num_key_value_heads=nkvh,
             head_dim=head_dim,
             intermediate_size=int(cfg["intermediate_size"]),
-            max_position_embeddings=int(max_tokens if max_tokens is not None
-                                        else cfg["max_position_embeddings"]),
+            max_position_embeddings=int(cfg["max_position_embeddings"]),
+            context_cap=int(max_tokens) if max_tokens is not None else None,
             rms_norm_eps=float(cfg["rms_norm_eps"]),
             rope_theta=float(cfg.get("rope_theta", 100000.0)),
             rope_scaling=rope_scaling,
@@ -134,6 +138,10 @@ class MiniCPMConfig:
         for k in pos:
             if getattr(self, k) <= 0:
                 raise ConfigError("%s must be positive, got %r" % (k, getattr(self, k)))
+        if self.context_cap is not None and self.context_cap <= 0:
+            raise ConfigError("max_tokens (the cap on the context) must be positive, got %r" % (self.context_cap,))
+        if self.torch_dtype not in ("bfloat16", "float32", "float16"):
+            raise ConfigError("torch_dtype %r: bfloat16, float32 or float16 expected" % (self.torch_dtype,))
         if self.num_attention_heads % self.num_key_value_heads:
             raise ConfigError("num_attention_heads (%d) is not a multiple of num_key_value_heads (%d)"
                               % (self.num_attention_heads, self.num_key_value_heads))
@@ -160,6 +168,18 @@ class MiniCPMConfig:
                 raise ConfigError("original_max_position_embeddings must be positive")
 
     # ---- derived constants -------------------------------------------------
+    @property
+    def max_positions(self) -> int:
+        """Positions a request may reach: the cap when one is given (jiuge.py:128-130), else the
+        checkpoint's max_position_embeddings."""
+        return self.context_cap if self.context_cap is not None else self.max_position_embeddings
+
+    @property
+    def default_dtype(self) -> str:
+        """The compute dtype to use when the caller names none: the checkpoint's torch_dtype;
+        float16 checkpoints run in bfloat16 (the kernels take bfloat16 and float32)."""
+        return "float32" if self.torch_dtype == "float32" else "bfloat16"
+
     @property
     def residual_scale(self) -> float:
         """scale_depth / sqrt(num_hidden_layers) on each branch (jiuge.py:109-114)."""
@@ -214,7 +234,8 @@ class MiniCPMConfig:
         rotary = PartSpec("rotary", "", {
             "head_dim": self.head_dim,
             "theta": self.rope_theta,
-            "max_positions": self.max_position_embeddings,
+            "max_positions": self.max_positions,
+            "model_max_positions": self.max_position_embeddings,
             "scaling": asdict(self.rope_scaling) if self.rope_scaling else None,
         })
         layers = []
@@ -243,7 +264,7 @@ class MiniCPMConfig:
             architecture=self.model_type,
             vocab_size=self.vocab_size,
             hidden_size=self.hidden_size,
-            max_positions=self.max_position_embeddings,
+            max_positions=self.max_positions,
             embedding=PartSpec("embedding", "model.embed_tokens.", {
                 "vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
                 "scale": self.scale_emb, "fallback_name": "lm_head."}),
@@ -253,7 +274,8 @@ class MiniCPMConfig:
                 "size": self.hidden_size, "eps": self.rms_norm_eps}),
             head=PartSpec("lm_head", "lm_head.", {
                 "vocab_size": self.vocab_size, "hidden_size": self.hidden_size,
-                "logit_scale": self.logit_scale, "fallback_name": "model.embed_tokens."}),
+                "logit_scale": self.logit_scale, "fallback_name": "model.embed_tokens.",
+                "tied": bool(self.tie_word_embeddings)}),
             eos_token_ids=list(self.eos_token_id),
             bos_token_id=self.bos_token_id,
         )

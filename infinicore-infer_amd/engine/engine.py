@@ -13,7 +13,7 @@ from typing import Dict, List, Optional, Sequence
 import numpy as np
 import torch
 
-from ..cache import CacheManager, CacheStorage, GroupSpec, OutOfPages
+from ..cache import CacheManager, CacheStorage, GroupSpec, OutOfPages, PositionOverflow
 from ..config import config_from_dir
 from ..kernels import ops
 from ..parts import Runtime, build_model
@@ -97,8 +97,11 @@ class Engine:
         self.groups: List[GroupSpec] = [
             GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots))
             for (nkv, dh, w), slots in keyed.items()]
+        # positions a request may reach: the model's limit and that of every part (a table's length)
+        limits = [model.spec.max_positions] + [p.position_limit() for p in model.all_parts()]
+        self.max_positions = min(int(l) for l in limits if l is not None)
         self.cache = CacheManager(self.groups, [self.num_pages] * len(self.groups), self.page_size,
-                                  self.max_requests, model.spec.max_positions)
+                                  self.max_requests, self.max_positions)
         self.storage = CacheStorage(self.groups, [self.num_pages] * len(self.groups), self.page_size,
                                     self.runtime.dtype, self.device)
         for slot, need in enumerate(needs):
@@ -120,10 +123,13 @@ class Engine:
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
-    def from_dir(cls, model_dir: str, dtype=torch.bfloat16, device="cuda:0", max_tokens: Optional[int] = None,
+    def from_dir(cls, model_dir: str, dtype=None, device="cuda:0", max_tokens: Optional[int] = None,
                  attention_impl: str = "auto", gemm_impl: str = "auto", max_context: Optional[int] = None,
                  **kw):
+        """``dtype`` None: the checkpoint's own (config.json's torch_dtype; float16 runs as bfloat16)."""
         cfg = config_from_dir(model_dir, max_tokens=max_context) if max_context else config_from_dir(model_dir)
+        if dtype is None:
+            dtype = getattr(torch, getattr(cfg, "default_dtype", "bfloat16"))
         rt = Runtime(dtype=dtype, device=device, attention_impl=attention_impl, gemm_impl=gemm_impl)
         model = build_model(cfg.model_spec(), rt)
         model.load_from_dir(model_dir)
@@ -171,8 +177,15 @@ class Engine:
                 if not (0 <= int(w) < len(e.tokens)):
                     raise ValueError("wanted place %r of request %r is outside its %d tokens" % (w, e.req_id, len(e.tokens)))
 
-        # ---- room in the cache: all or nothing ------------------------------------------------
+        # ---- room in the cache and in the positions: all or nothing -------------------------------
+        # Everything that can refuse the step is looked at for ALL entries before anything changes.
         new_ids = [e.req_id for e in entries if not self.cache.has_request(e.req_id)]
+        before = {e.req_id: (self.cache.length(e.req_id) if self.cache.has_request(e.req_id) else 0)
+                  for e in entries}
+        for e in entries:
+            if before[e.req_id] + len(e.tokens) > self.max_positions:
+                raise PositionOverflow("request %r would reach position %d, the model ends at %d"
+                                       % (e.req_id, before[e.req_id] + len(e.tokens), self.max_positions))
         if len(new_ids) > self.cache.slots.n_free:
             raise OutOfPages("%d new requests but %d free state slots" % (len(new_ids), self.cache.slots.n_free))
         need = [0] * len(self.groups)
@@ -185,17 +198,29 @@ class Engine:
         for g, n in enumerate(need):
             if n > self.cache.free_pages(g):
                 raise OutOfPages("step needs %d pages of group %d, %d free" % (n, g, self.cache.free_pages(g)))
-        for rid in new_ids:
-            self.add_request(rid)
-        starts = [self.cache.append(e.req_id, len(e.tokens)) for e in entries]
 
-        if (self.use_graphs and len(entries) <= self.graph_max_batch
-                and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
-            logits = self._graph_step(entries, starts)
-        else:
-            ctx = self._build_context(entries, starts)
-            with ops.stream_scope():
-                logits = self.model.forward(ctx)
+        # From here on the cache changes.  Should anything still fail (an allocation, a kernel that
+        # refuses its arguments), the cache is put back: lengths, pages and newly admitted requests.
+        # What a failed forward wrote lies beyond every request's length and is never read.
+        try:
+            for rid in new_ids:
+                self.add_request(rid)
+            starts = [self.cache.append(e.req_id, len(e.tokens)) for e in entries]
+            if (self.use_graphs and len(entries) <= self.graph_max_batch
+                    and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
+                logits = self._graph_step(entries, starts)
+            else:
+                ctx = self._build_context(entries, starts)
+                with ops.stream_scope():
+                    logits = self.model.forward(ctx)
+        except BaseException:
+            for e in entries:
+                if e.req_id in new_ids:
+                    if self.cache.has_request(e.req_id):
+                        self.cache.release(e.req_id)
+                elif self.cache.length(e.req_id) != before[e.req_id]:
+                    self.cache.truncate(e.req_id, before[e.req_id])
+            raise
         for e in entries:
             self.cache.trim(e.req_id)
         self.steps_run += 1

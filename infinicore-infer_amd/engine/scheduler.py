@@ -224,15 +224,22 @@ class Scheduler:
                 out.append((t, int(tok)))
                 if tok in t.end_tokens:
                     self._finish(r, "stop")
-                elif t.pos >= t.max_tokens:
-                    self._finish(r, "length")
+                elif t.pos >= t.max_tokens or (self.cache.max_positions is not None
+                                               and t.pos >= self.cache.max_positions):
+                    self._finish(r, "length")       # the task's own limit, or the model has no position left
                 elif t.max_new_tokens is not None and len(t.generated) >= t.max_new_tokens:
                     self._finish(r, "length")
         return out
 
-    def run(self) -> List[InferTask]:
-        """Step until every request has finished."""
+    def run(self, on_step=None) -> List[InferTask]:
+        """Step until every request has finished.  ``on_step(new, seconds)``, when given, is called
+        after every step with its (task, token) pairs and the time the step took on the host clock
+        (a step that samples ends with the copy of its tokens to the host, so that is its whole time)."""
+        import time
         while self.has_unfinished():
-            self.step()
+            t0 = time.perf_counter()
+            new = self.step()
+            if on_step is not None:
+                on_step(new, time.perf_counter() - t0)
         done, self.finished = self.finished, []
         return done

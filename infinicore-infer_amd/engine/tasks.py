@@ -11,6 +11,8 @@ here a request id of the engine's paged cache instead of a whole-context slab
 import itertools
 from typing import List, Optional, Sequence
 
+from ..sampling.params import SamplingParams
+
 _next_handle = itertools.count()
 
 
@@ -38,6 +40,7 @@ class KVCache:
 class InferTask:
     def __init__(self, id, tokens, max_tokens, temperature=1.0, topk=1, topp=1.0, end_tokens=(),
                  seed: int = 0, max_new_tokens: Optional[int] = None):
+        SamplingParams(temperature, topk, topp, seed)      # refuses a negative temperature, topp outside [0, 1], ...
         self.id = id
         self.finish_reason = None
         self.tokens = list(tokens)             # tokens to feed in the next step

@@ -52,23 +52,29 @@ class Attention(Mixer):
     # ---- weights: names of scripts/jiuge.py:45-63 ------------------------------
     def weight_specs(self):
         n = self.name
+        pack = None if self.shared_kv else n + "qkv_proj.packed"
         specs = {
-            n + "q_proj.weight": WeightSpec((self.nh * self.dh, self.hidden_size)),
+            n + "q_proj.weight": WeightSpec((self.nh * self.dh, self.hidden_size), pack=pack and (pack, 0)),
             n + "o_proj.weight": WeightSpec((self.hidden_size, self.nh * self.dh)),
         }
         if not self.shared_kv:
-            specs[n + "k_proj.weight"] = WeightSpec((self.nkvh * self.dh, self.hidden_size))
-            specs[n + "v_proj.weight"] = WeightSpec((self.nkvh * self.dh, self.hidden_size))
+            specs[n + "k_proj.weight"] = WeightSpec((self.nkvh * self.dh, self.hidden_size), pack=(pack, 1))
+            specs[n + "v_proj.weight"] = WeightSpec((self.nkvh * self.dh, self.hidden_size), pack=(pack, 2))
         return specs
 
     def load_weights(self, tensors):
         n = self.name
         names = ["q_proj.weight"] + ([] if self.shared_kv else ["k_proj.weight", "v_proj.weight"])
         mats = [tensors[n + s] for s in names]
-        if len({m.dtype for m in mats}) > 1:
-            mats = [m.to(torch.float32) for m in mats]
-        # rows [Q; K; V] of one fused projection (jiuge.py:237-239), unpermuted
-        self.w_qkv = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
+        # rows [Q; K; V] of one fused projection (jiuge.py:237-239), unpermuted.  The loader lays the
+        # three out one after the other and hands out their concatenation; otherwise copy them together.
+        packed = tensors.get(n + "qkv_proj.packed")
+        if packed is not None:
+            self.w_qkv = packed
+        else:
+            if len({m.dtype for m in mats}) > 1:
+                mats = [m.to(torch.float32) for m in mats]
+            self.w_qkv = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
         self.w_o = tensors[n + "o_proj.weight"]
 
     # ---- forward ---------------------------------------------------------------------

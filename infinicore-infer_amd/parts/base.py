@@ -135,6 +135,11 @@ class Part:
     def sub_parts(self):
         return ()
 
+    def position_limit(self):
+        """Positions this part can take (a table's length), or None when it has no limit.  The
+        engine refuses a step that would go beyond the smallest limit before it changes anything."""
+        return None
+
 
 class Norm(Part):
     category = "norm"

@@ -40,6 +40,16 @@ class Embedding(Part):
         return ops.embed(tokens, self.table, x, self.scale)
 
 
+class _ScaledNorm:
+    """(weight, eps) of a norm whose weight already carries the head's scale."""
+
+    def __init__(self, weight, eps):
+        self._d = (weight, eps)
+
+    def deferred(self):
+        return self._d
+
+
 @register_part("head", "lm_head")
 class LMHead(Part):
     graph_safe = True
@@ -48,25 +58,42 @@ class LMHead(Part):
     category = "head"
 
     def __init__(self, name, runtime, vocab_size: int, hidden_size: int, logit_scale: float = 1.0,
-                 fallback_name=None):
+                 fallback_name=None, tied: bool = False):
         super().__init__(name, runtime)
         self.vocab_size, self.hidden_size = vocab_size, hidden_size
         self.logit_scale = float(logit_scale)
         self.fallback = fallback_name + "weight" if fallback_name else None
+        self.tied = bool(tied) and self.fallback is not None
         self.weight = None
+        self._scaled_norms = {}
 
     def weight_specs(self):
-        return {self.name + "weight": WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback)}
+        return {self.name + "weight": WeightSpec((self.vocab_size, self.hidden_size), "matrix", self.fallback,
+                                                 tied=self.tied)}
 
     def load_weights(self, tensors):
         self.weight = tensors[self.name + "weight"]
+        self._scaled_norms = {}
+
+    def deferred_norm(self, final_norm):
+        """The final norm as the last block's successor when its rows reach the head half done: its
+        weight times the logit scale, so that the scale enters before the rounding to the compute
+        dtype exactly as on the other path (``out_scale`` of the norm kernel; the reference scales
+        the norm's weight, scripts/jiuge.py:198-201).  None when the norm cannot be split."""
+        d = final_norm.deferred()
+        if d is None:
+            return None
+        key = id(final_norm)
+        if key not in self._scaled_norms:
+            self._scaled_norms[key] = _ScaledNorm((d[0] * self.logit_scale).contiguous(), d[1])
+        return self._scaled_norms[key]
 
     def forward(self, x, rows, final_norm, ctx):
         """Float32 logits [len(rows), vocab] of the residual rows ``rows``."""
         if isinstance(x, DeferredRows):
             # every row in order, the final norm half done: its row factors go into the product
             logits = ctx.ws.buffer("logits", (x.shape[0], self.vocab_size), torch.float32)
-            return linear(x, self.weight, logits, self.runtime.gemm_impl, alpha=self.logit_scale)
+            return linear(x, self.weight, logits, self.runtime.gemm_impl)     # the scale is in x (deferred_norm)
         n = rows.numel()
         h = ctx.ws.buffer("head_in", (n, self.hidden_size), self.runtime.dtype)
         final_norm.forward(x, h, rows=rows, out_scale=self.logit_scale)

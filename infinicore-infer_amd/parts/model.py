@@ -51,6 +51,22 @@ class DecoderModel:
             if not e.writes_cache and e.cache not in writers:
                 raise ValueError("cache slot %d is read but never written" % e.cache)
         self._writers = writers
+        # an entry that reads another entry's cache must fit what the writer keeps: the same heads and
+        # head size, and no more keys than the writer's window holds (pages behind a window are given
+        # back and their block-table entries are reused)
+        for e in self.schedule:
+            if e.writes_cache:
+                continue
+            wn = self.layers[writers[e.cache]].mixer.cache_need()
+            rn = self.layers[e.layer].mixer.cache_need()
+            if wn.kind != "kv" or rn.kind != "kv":
+                continue
+            if (rn.n_kv_heads, rn.head_dim) != (wn.n_kv_heads, wn.head_dim):
+                raise ValueError("layer %d reads cache slot %d with %d kv heads of %d, its writer (layer %d) keeps %d of %d"
+                                 % (e.layer, e.cache, rn.n_kv_heads, rn.head_dim, writers[e.cache], wn.n_kv_heads, wn.head_dim))
+            if wn.window and (not rn.window or rn.window > wn.window):
+                raise ValueError("layer %d reads cache slot %d over %s keys, its writer (layer %d) keeps a window of %d"
+                                 % (e.layer, e.cache, rn.window or "all", writers[e.cache], wn.window))
 
     # ---- parts and weights ---------------------------------------------------------
     def all_parts(self):
@@ -124,7 +140,7 @@ class DecoderModel:
             if i < last:
                 successor = self.layers[self.schedule[i + 1].layer].entry_norm()
             elif ctx.want_rows_identity and getattr(self.head, "accepts_deferred", False):
-                successor = self.final_norm
+                successor = self.head.deferred_norm(self.final_norm)
             else:
                 successor = None
             pending = block.forward(x, pending, ctx, ctx.cache_view(e), successor=successor)

@@ -8,8 +8,9 @@ of the checkpoint's own row order, which is what the kernel does, so weights
 load unpermuted.  Tables are built in float64 and held in float32.
 
 Long-context scaling ("longrope", not in the reference): each pair's frequency
-is divided by a factor from the long array when the configured context exceeds
-the original one, else from the short array; cos and sin are multiplied by
+is divided by a factor from the long array when the checkpoint's context
+(max_position_embeddings, not a serving cap on it) exceeds the original one, else
+from the short array; cos and sin are multiplied by
 sqrt(1 + ln(ratio) / ln(original)) when ratio = context / original > 1.
 """
 import math
@@ -21,15 +22,20 @@ from .base import DeferredRows, PositionEncoding, register_part
 from .linear import FEW_ROWS
 
 
-def rotary_tables(head_dim, theta, max_positions, scaling=None, rot_dim=None):
+def rotary_tables(head_dim, theta, max_positions, scaling=None, rot_dim=None, model_max_positions=None):
+    """cos and sin [max_positions, rot/2] in float32.  ``max_positions`` is only the tables' length;
+    long-context scaling (which factor array, the magnitude) follows ``model_max_positions``, the
+    checkpoint's own context length, so a serving cap on the context changes no value."""
     rot = head_dim if rot_dim is None else rot_dim
+    if model_max_positions is None:
+        model_max_positions = max_positions
     half = rot // 2
     j = torch.arange(half, dtype=torch.float64)
     inv_freq = 1.0 / torch.pow(torch.tensor(float(theta), dtype=torch.float64), j / half)
     magnitude = 1.0
     if scaling:
         orig = int(scaling["original_max_position_embeddings"])
-        ratio = max_positions / orig
+        ratio = model_max_positions / orig
         if ratio > 1.0:
             factors = scaling["long_factor"]
             magnitude = math.sqrt(1.0 + math.log(ratio) / math.log(orig))
@@ -48,18 +54,22 @@ class Rotary(PositionEncoding):
     graph_safe = True
 
     def __init__(self, name, runtime, head_dim: int, theta: float, max_positions: int, scaling=None,
-                 rot_dim=None):
+                 rot_dim=None, model_max_positions=None):
         super().__init__(name, runtime)
         self.head_dim = head_dim
         self.rot_dim = head_dim if rot_dim is None else rot_dim
         if self.rot_dim % 2 or self.rot_dim > head_dim:
             raise ValueError("rotary: rot_dim must be even and at most head_dim")
         self.max_positions = max_positions
-        key = (head_dim, float(theta), max_positions, repr(scaling), self.rot_dim, str(runtime.device))
+        key = (head_dim, float(theta), max_positions, repr(scaling), self.rot_dim, model_max_positions,
+               str(runtime.device))
         if key not in _TABLES:            # layers with the same parameters share one pair of tables
-            cos, sin = rotary_tables(head_dim, theta, max_positions, scaling, self.rot_dim)
+            cos, sin = rotary_tables(head_dim, theta, max_positions, scaling, self.rot_dim, model_max_positions)
             _TABLES[key] = (cos.to(runtime.device).contiguous(), sin.to(runtime.device).contiguous())
         self.cos, self.sin = _TABLES[key]
+
+    def position_limit(self):
+        return self.max_positions
 
     def rotate_and_store(self, qkv, ctx, cache, n_heads, n_kv_heads, head_dim):
         if ctx.max_position >= self.max_positions:

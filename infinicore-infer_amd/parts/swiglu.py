@@ -29,17 +29,21 @@ class SwiGLU(FeedForward):
     def weight_specs(self):
         n, d, di = self.name, self.hidden_size, self.intermediate_size
         return {
-            n + "gate_proj.weight": WeightSpec((di, d)),
-            n + "up_proj.weight": WeightSpec((di, d)),
+            n + "gate_proj.weight": WeightSpec((di, d), pack=(n + "gate_up_proj.packed", 0)),
+            n + "up_proj.weight": WeightSpec((di, d), pack=(n + "gate_up_proj.packed", 1)),
             n + "down_proj.weight": WeightSpec((d, di)),
         }
 
     def load_weights(self, tensors):
         n = self.name
-        g, u = tensors[n + "gate_proj.weight"], tensors[n + "up_proj.weight"]
-        if g.dtype != u.dtype:
-            g, u = g.to(torch.float32), u.to(torch.float32)
-        self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
+        packed = tensors.get(n + "gate_up_proj.packed")      # laid out [gate; up] by the loader
+        if packed is not None:
+            self.w_gate_up = packed
+        else:
+            g, u = tensors[n + "gate_proj.weight"], tensors[n + "up_proj.weight"]
+            if g.dtype != u.dtype:
+                g, u = g.to(torch.float32), u.to(torch.float32)
+            self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = tensors[n + "down_proj.weight"]
 
     def forward(self, h, ctx, tail=None):

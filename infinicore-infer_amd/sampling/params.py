@@ -21,12 +21,12 @@ class SamplingParams:
     seed: int = 0
 
     def __post_init__(self):
-        if self.temperature < 0:
-            raise ValueError("temperature must be >= 0")
-        if self.topk < 0:
-            raise ValueError("topk must be >= 0 (0 keeps every token)")
+        if not (self.temperature >= 0) or self.temperature == float("inf"):
+            raise ValueError("temperature must be a finite number >= 0, got %r" % (self.temperature,))
+        if int(self.topk) != self.topk or self.topk < 0:
+            raise ValueError("topk must be an integer >= 0 (0 keeps every token), got %r" % (self.topk,))
         if not (0.0 <= self.topp <= 1.0):
-            raise ValueError("topp must lie in [0, 1]")
+            raise ValueError("topp must lie in [0, 1], got %r" % (self.topp,))
 
     @property
     def greedy(self) -> bool:

@@ -81,12 +81,19 @@ def test_random_orders_conserve_pages(seed):
         elif op < 0.8 and live:
             r = rng.choice(live)
             k = rng.choice([1, 1, 1, 2, 7, 16, 33])
+            before = (m.length(r), m.free_pages(0), m.free_pages(1), [list(t) for t in m.requests[r].tables])
             try:
                 m.append(r, k)
-                m.trim(r)
-            except (OutOfPages, PositionOverflow):
-                before = (m.length(r), m.free_pages(0), m.free_pages(1))
-                assert before == (m.length(r), m.free_pages(0), m.free_pages(1))
+            except (OutOfPages, PositionOverflow):       # a refused append changes nothing
+                assert before == (m.length(r), m.free_pages(0), m.free_pages(1),
+                                  [list(t) for t in m.requests[r].tables])
+            else:
+                if rng.random() < 0.15:                  # a step that failed after its appends is undone
+                    m.truncate(r, before[0])
+                    assert before == (m.length(r), m.free_pages(0), m.free_pages(1),
+                                      [list(t) for t in m.requests[r].tables])
+                else:
+                    m.trim(r)
         elif live:
             r = live.pop(rng.randrange(len(live)))
             m.release(r)
@@ -97,3 +104,21 @@ def test_random_orders_conserve_pages(seed):
         m.release(r)
     m.check_invariants()
     assert m.free_pages(0) == 24 and m.free_pages(1) == 24 and m.slots.n_free == 5
+
+
+def test_truncate_gives_back_exactly_what_the_appends_took():
+    m = CacheManager([FULL], [8], 16, max_requests=2, max_positions=200)
+    m.admit("a")
+    m.append("a", 20)
+    table = list(m.block_table("a", 0))
+    m.append("a", 30)
+    m.append("a", 1)
+    assert m.free_pages(0) == 8 - 4
+    m.truncate("a", 20)
+    assert m.length("a") == 20 and m.block_table("a", 0) == table and m.free_pages(0) == 6
+    m.check_invariants()
+    m.truncate("a", 0)
+    assert m.block_table("a", 0) == [] and m.free_pages(0) == 8
+    with pytest.raises(Exception):
+        m.truncate("a", 5)                      # it cannot grow a request
+    m.check_invariants()

@@ -87,6 +87,35 @@ def test_round_trip_through_a_folder(tmp_path):
     (tmp_path / "config.json").write_text(json.dumps(c.to_dict()))
     c2 = config_from_dir(str(tmp_path))
     assert c2 == c
-    assert config_from_dir(str(tmp_path), max_tokens=99).max_position_embeddings == 99     # jiuge.py:128-130
+    capped = config_from_dir(str(tmp_path), max_tokens=99)                                 # jiuge.py:128-130
+    assert capped.max_positions == 99 and capped.model_spec().max_positions == 99
+    assert capped.max_position_embeddings == 512 and c.max_positions == 512
     with pytest.raises(ConfigError):
         config_from_dir(str(tmp_path / "nowhere"))
+
+
+def test_a_cap_on_the_context_changes_no_rotary_value():
+    """The cap bounds positions and table length; which longrope factors apply and the magnitude of
+    cos/sin follow the checkpoint's own context length.  (TINY_C: 512 configured, 128 original, so the
+    long factors and a magnitude above 1 apply; a cap of 100 lies below the original length.)"""
+    import torch
+    from infinicore_infer_amd.parts.rotary import rotary_tables
+    full = config_from_dict(H.TINY_C).model_spec().layers[0].mixer.params["position_encoding"].params
+    capped = config_from_dict(H.TINY_C, max_tokens=100).model_spec().layers[0].mixer.params["position_encoding"].params
+    assert capped["max_positions"] == 100 and capped["model_max_positions"] == 512
+    cos_f, sin_f = rotary_tables(**full)
+    cos_c, sin_c = rotary_tables(**capped)
+    assert cos_c.shape[0] == 100
+    assert torch.equal(cos_c, cos_f[:100]) and torch.equal(sin_c, sin_f[:100])
+    assert float(cos_f[0].max()) > 1.0                      # the magnitude factor is in
+    # what the mistake would give: factors and magnitude chosen from the cap
+    cos_w, _ = rotary_tables(**dict(capped, model_max_positions=100))
+    assert not torch.equal(cos_w, cos_c)
+
+
+def test_torch_dtype_names_the_default_compute_dtype():
+    assert config_from_dict(H.TINY_A).default_dtype == "bfloat16"
+    assert config_from_dict(dict(H.TINY_A, torch_dtype="float32")).default_dtype == "float32"
+    assert config_from_dict(dict(H.TINY_A, torch_dtype="float16")).default_dtype == "bfloat16"
+    with pytest.raises(ConfigError):
+        config_from_dict(dict(H.TINY_A, torch_dtype="int8"))

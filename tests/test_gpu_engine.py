@@ -68,14 +68,6 @@ def test_replay_modes(tmp_path_factory, name, dname, dtype, tol, mode):
 
 
 @pytest.mark.parametrize("dname,dtype,tol", DTYPES)
-def test_mixed_reuses_pages(tmp_path_factory, dname, dtype, tol):
-    """The mixed trace's pool is smaller than what all requests would need together."""
-    requests = _requests("B")
-    steps, max_tokens = H.trace_mixed(requests)
-    assert max_tokens < sum(H.ceil64(len(t)) for t in requests.values())
-
-
-@pytest.mark.parametrize("dname,dtype,tol", DTYPES)
 @pytest.mark.parametrize("page_size", [16, 64])
 def test_generic_attention_path(tmp_path_factory, dname, dtype, tol, page_size):
     """The general attention kernel alone (tiled kernels off) on the head-size-64 model."""

@@ -181,3 +181,45 @@ def test_sampling_draws_do_not_depend_on_preemption():
     assert not SamplingParams(temperature=0.8, topk=50).greedy
     with pytest.raises(ValueError):
         SamplingParams(topp=1.5)
+    for bad in (dict(temperature=-0.5), dict(temperature=float("nan")), dict(topk=-1), dict(topp=-0.1), dict(topk=2.5)):
+        with pytest.raises(ValueError):
+            SamplingParams(**bad)
+        with pytest.raises(ValueError):                  # a request's options are checked when it is made
+            InferTask("bad", [1, 2], 10, **bad)
+
+
+def test_a_task_whose_limit_lies_beyond_the_models_positions_ends_with_length():
+    """max_tokens of a task may exceed what the model can hold; decoding stops at the model's last
+    position with "length" instead of asking the step for a position that does not exist."""
+    eng = FakeEngine(num_pages=16, max_positions=24)
+    s = Scheduler(eng, max_batch_tokens=64, chunk_size=8)
+    t = InferTask("t", list(range(10)), max_tokens=10 ** 6, end_tokens=[])
+    s.add(t)
+    s.run()                                              # FakeEngine.step would raise PositionOverflow
+    assert t.finish_reason == "length" and t.pos == 24
+    assert t.generated == _expected(range(10), 24 - 10 + 1)
+    assert eng.cache.free_pages() == 16
+    long = InferTask("long", list(range(30)), max_tokens=10 ** 6)     # the prompt alone is too long
+    s.add(long)
+    s.run()
+    assert long.finish_reason == "length" and long.generated == []
+
+
+def test_command_line_arguments():
+    """The command line's surface: the reference's positional form (scripts/jiuge.py:646-677) and the
+    options beside it; parsing needs no GPU."""
+    from infinicore_infer_amd.minicpm import _parse
+    path, ndev, a = _parse(["--amd", "/m", "1", "--prompt-ids", "1,2", "--prompt-ids", "3", "--max-new-tokens", "4",
+                            "--top-k", "5", "--top-p", "0.5", "--chunk-size", "8", "--max-batch-tokens", "16",
+                            "--num-pages", "9", "--page-size", "32", "--dtype", "float32"])
+    assert (path, ndev) == ("/m", 1)
+    assert a.prompt_ids == ["1,2", "3"] and a.max_new_tokens == 4 and a.topk == 5 and a.topp == 0.5
+    assert (a.chunk_size, a.max_batch_tokens, a.num_pages, a.page_size, a.dtype) == (8, 16, 9, 32, "float32")
+    path, ndev, a = _parse(["--random-weights", "--config", "c.json", "--prompt-len", "12", "--num-prompts", "3",
+                            "--topk", "2", "--max-steps", "6"])
+    assert path is None and a.random_weights and a.config == "c.json" and a.prompt_len == 12 and a.num_prompts == 3
+    assert a.topk == 2 and a.max_new_tokens == 6 and a.dtype is None
+    for bad in (["--nvidia", "/m"], [], ["/m", "--random-weights", "--config", "c"], ["--random-weights"],
+                ["/m", "--device", "cpu"]):
+        with pytest.raises(SystemExit):
+            _parse(bad)

@@ -120,3 +120,89 @@ def test_random_weights_from_the_command_line(tmp_path):
     a, b = load_file(str(out / "model.safetensors")), load_file(os.path.join(ref, "model.safetensors"))
     assert sorted(a) == sorted(b) and all(torch.equal(a[k], b[k]) for k in a)
     assert json.load(open(out / "config.json"))["vocab_size"] == H.TINY_B["vocab_size"]
+
+
+def test_unexpected_dtypes_are_refused_by_tensor_name(tmp_path):
+    """A matrix or a norm weight stored as integers or 8-bit floats (a quantized checkpoint) is an
+    error that names the tensor, together with whatever else is wrong."""
+    folder = H.make_model_dir(tmp_path, "A", seed=3)
+    path = os.path.join(folder, "model.safetensors")
+    sd = load_file(path)
+    sd["model.layers.0.mlp.up_proj.weight"] = torch.zeros(160, 64, dtype=torch.int8)
+    sd["model.layers.1.input_layernorm.weight"] = torch.ones(64, dtype=torch.int32)
+    if hasattr(torch, "float8_e4m3fn"):
+        sd["model.layers.1.self_attn.o_proj.weight"] = torch.zeros(64, 64).to(torch.float8_e4m3fn)
+    del sd["model.norm.weight"]
+    save_file(sd, path)
+    with pytest.raises(WeightError) as e:
+        _model("A").load_from_dir(folder)
+    names = [w[0] for w in e.value.wrong_dtype]
+    assert "model.layers.0.mlp.up_proj.weight" in names and "model.layers.1.input_layernorm.weight" in names
+    assert e.value.missing == ["model.norm.weight"]
+    msg = str(e.value)
+    assert "I8" in msg and "I32" in msg and "up_proj" in msg
+    if hasattr(torch, "float8_e4m3fn"):
+        assert "model.layers.1.self_attn.o_proj.weight" in names
+    # float16 is a floating-point type: converted to the compute dtype, not refused
+    folder2 = H.make_model_dir(tmp_path, "B", seed=3)
+    sd = load_file(os.path.join(folder2, "model.safetensors"))
+    sd = {k: v.to(torch.float16) for k, v in sd.items()}
+    save_file(sd, os.path.join(folder2, "model.safetensors"))
+    m = _model("B")
+    m.load_from_dir(folder2)
+    assert m.layers[0].mixer.w_o.dtype == torch.bfloat16 and m.final_norm.weight.dtype == torch.float32
+
+
+def test_tied_in_the_configuration_but_both_tensors_present(tmp_path):
+    """Presence decides which tensor backs which table (scripts/jiuge.py:182-191).  When the
+    configuration ties them and the files still hold both: equal tensors are kept once, different ones
+    are an error (one of them would silently be ignored otherwise)."""
+    folder = H.make_model_dir(tmp_path, "A", seed=4)
+    path = os.path.join(folder, "model.safetensors")
+    sd = load_file(path)
+    sd["lm_head.weight"] = sd["model.embed_tokens.weight"].clone()
+    save_file(sd, path)
+    m = _model("A")
+    m.load_from_dir(folder)
+    assert m.head.weight is m.embedding.table or m.head.weight.data_ptr() == m.embedding.table.data_ptr()
+    sd["lm_head.weight"] = sd["model.embed_tokens.weight"] * 2
+    save_file(sd, path)
+    with pytest.raises(WeightError) as e:
+        _model("A").load_from_dir(folder)
+    assert "lm_head.weight" in str(e.value) and "differ" in str(e.value)
+    # not tied in the configuration: both are used as they are
+    cfg = dict(H.TINY_A, tie_word_embeddings=False)
+    m2 = build_model(config_from_dict(cfg).model_spec(), Runtime(torch.bfloat16, "cpu"))
+    m2.load_from_dir(folder)
+    assert torch.equal(m2.head.weight, sd["lm_head.weight"]) and torch.equal(m2.embedding.table, sd["model.embed_tokens.weight"])
+
+
+def test_one_allocation_and_fused_projections_without_a_copy(tmp_path):
+    """All tensors are views of one allocation; q, k, v (and gate, up) lie one after the other, so the
+    fused projection matrices are views too and equal the concatenation of the stored tensors."""
+    from infinicore_infer_amd.weights import loader
+    folder = H.make_model_dir(tmp_path, "C", seed=7)
+    sd = load_file(os.path.join(folder, "model.safetensors"))
+    m = _model("C")
+    m.load_from_dir(folder)
+    base = m.embedding.table.untyped_storage().data_ptr()
+    for p in m.all_parts():
+        for k, v in vars(p).items():
+            if isinstance(v, torch.Tensor) and k not in ("cos", "sin"):      # rotary tables are no weights
+                assert v.untyped_storage().data_ptr() == base
+                assert (v.data_ptr() - base) % 256 == 0        # every tensor (and pack) starts on a 256-byte boundary
+    for i, layer in enumerate(m.layers):
+        n = "model.layers.%d." % i
+        want = torch.cat([sd[n + "self_attn.%s_proj.weight" % x] for x in "qkv"], 0)
+        assert torch.equal(layer.mixer.w_qkv, want) and layer.mixer.w_qkv.is_contiguous()
+        want = torch.cat([sd[n + "mlp.gate_proj.weight"], sd[n + "mlp.up_proj.weight"]], 0)
+        assert torch.equal(layer.feed_forward.w_gate_up, want)
+        assert torch.equal(layer.mixer_norm.weight, sd[n + "input_layernorm.weight"].float())
+    assert loader.last_load_report["bytes"] >= sum(v.numel() * 2 for v in sd.values())
+    assert loader.last_load_report["seconds"] > 0
+    # q stored in 32-bit, k and v not: no common layout, the part copies them together in float32
+    sd["model.layers.0.self_attn.q_proj.weight"] = sd["model.layers.0.self_attn.q_proj.weight"].float()
+    save_file(sd, os.path.join(folder, "model.safetensors"))
+    m = _model("C")
+    m.load_from_dir(folder)
+    assert m.layers[0].mixer.w_qkv.dtype == torch.float32 and m.layers[1].mixer.w_qkv.dtype == torch.bfloat16
