@@ -84,6 +84,7 @@ class StepContext:
         self.max_context = 0             # most keys any single-token row sees
         self.cu_count = 256              # compute units, for split heuristics
         self.fixed_decode_splits: Optional[int] = None
+        self.group_views = []            # per cache group: (slots int32 [T], block tables int32 [R, max_blocks])
         self._views: Dict[int, LayerCacheView] = {}
 
     def cache_view(self, entry) -> LayerCacheView:
@@ -93,32 +94,12 @@ class StepContext:
         return v
 
     def decode_splits(self, n_kv_heads: int, window: int = 0, matrix_core_tiles_of: int = 0) -> int:
-        """How many ways to split the keys of single-token rows.  From sweeps on MI355X with a
-        cold cache.  One split writes the result itself; more cost a second kernel (about 5 us), so
-        short contexts are never split: up to 1,024 keys with one query head per kv head (a wave walks
-        keys with vector instructions), up to 256 with grouped query heads on the matrix cores
-        (``matrix_core_tiles_of`` = the head size; its blocks walk 128 keys a round).
-        Beyond that, one head per kv head: few (row, kv head) pairs want about 1.75 blocks per compute
-        unit but at least 384 keys a block; a middling number of pairs already draws the full
-        bandwidth unsplit up to 2,048 keys; many pairs want about 3.4 blocks per unit.  Grouped heads:
-        a wave has a whole 32-key tile in flight, so 128 / head size blocks per unit are enough and
-        more only add partial results to merge.  A split never gets fewer than 64 keys."""
+        """How many ways to split the keys of single-token rows: the kernel library's rule
+        (ic_attn_decode_splits, from sweeps on MI355X with a cold cache), so that steps issued from
+        Python and from native code split alike.  ``matrix_core_tiles_of``: the head size when the
+        grouped-query kernel runs, else 0."""
         if self.fixed_decode_splits is not None:
             return self.fixed_decode_splits
-        keys = self.max_context if not window else min(self.max_context, window)
-        base = max(1, self.n_decode_rows * n_kv_heads)
-        cu = self.cu_count
-        min_keys = 64
-        if matrix_core_tiles_of:
-            if keys <= 256:
-                return 1
-            per_unit = 128.0 / matrix_core_tiles_of
-        else:
-            if keys <= 1024 or (0.3 * cu <= base < 0.6 * cu and keys <= 2048):
-                return 1
-            if base < 0.3 * cu:
-                per_unit, min_keys = 1.75, 384
-            else:
-                per_unit = 1.75 if base < 0.6 * cu else 3.4
-        want = max(1, int(per_unit * cu / base + 0.5))
-        return int(max(1, min(want, max(1, keys // min_keys), 64)))
+        from ..kernels.lib import get_lib
+        return int(get_lib().ic_attn_decode_splits(self.n_decode_rows, n_kv_heads, int(window or 0), self.max_context,
+                                                   int(matrix_core_tiles_of), self.cu_count))

@@ -72,9 +72,12 @@ class _PinnedRing:
 
 class Engine:
     def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 64,
-                 num_pages: Optional[int] = None, use_graphs: bool = True, graph_max_batch: int = 64):
+                 num_pages: Optional[int] = None, use_graphs: bool = True, graph_max_batch: int = 64,
+                 use_native: bool = True):
         """``max_tokens``: the most tokens live requests hold at any time, each
-        request's count rounded up to whole pages; every group's pool is sized for it."""
+        request's count rounded up to whole pages; every group's pool is sized for it.
+        ``use_native``: let one native call issue a step's kernels when every part of the model
+        has a native description (otherwise, and for other models, the parts' Python forward runs)."""
         self.model = model
         self.runtime: Runtime = model.runtime
         self.device = torch.device(self.runtime.device)
@@ -120,6 +123,10 @@ class Engine:
         self.graph_max_batch = int(graph_max_batch)
         self._graphs: Dict[tuple, "_DecodeGraph"] = {}
         self.graph_replays = 0
+        # the step function in native code, when the model's parts all have a native description
+        from .native import NativeDecoder
+        self.native = NativeDecoder.try_build(self) if use_native else None
+        self.native_steps = 0
 
     # ---- construction -----------------------------------------------------------------
     @classmethod
@@ -212,7 +219,7 @@ class Engine:
             else:
                 ctx = self._build_context(entries, starts)
                 with ops.stream_scope():
-                    logits = self.model.forward(ctx)
+                    logits = self._forward(ctx)
         except BaseException:
             for e in entries:
                 if e.req_id in new_ids:
@@ -225,6 +232,21 @@ class Engine:
             self.cache.trim(e.req_id)
         self.steps_run += 1
         return logits
+
+    def _forward(self, ctx):
+        """The model's forward for a packed step: issued by one native call when the model allows it
+        (not while library products are being timed: that is done product by product from Python)."""
+        from ..parts import linear as _linear
+        if self.native is not None and not _linear.TUNE_LIBRARY:
+            try:
+                out = self.native.forward(ctx)
+                self.native_steps += 1
+                return out
+            except ops.NoLibraryAlgorithm:
+                # the library has no algorithm for a product of this step: the Python path knows a detour.
+                # Nothing of the half-issued step is kept (the residual stream is rebuilt, cache writes repeat).
+                self.native = None
+        return self.model.forward(ctx)
 
     # ---- packing the batch ------------------------------------------------------------------------
     def _build_context(self, entries, starts) -> StepContext:
@@ -322,6 +344,7 @@ class Engine:
         ctx.max_context = _context_bucket(max_ctx) if max_ctx else 0
         ctx.cu_count = self.cu_count
         group_views = [(view("slots%d" % g), view("tables%d" % g).view(R, group_maxb[g])) for g in range(n_groups)]
+        ctx.group_views = group_views
         for slot in range(self.model.spec.num_cache_slots()):
             if slot in self._slot_group:
                 slots, tables_g = group_views[self._slot_group[slot]]
@@ -443,6 +466,7 @@ class _DecodeGraph:
         ctx.req_len = [1] * R
         ctx.max_context = ctx_bucket
         ctx.cu_count = engine.cu_count
+        ctx.group_views = [(view("slots%d" % g), view("tables%d" % g).view(R, self.maxb)) for g in range(ng)]
         for slot in range(engine.model.spec.num_cache_slots()):
             if slot in engine._slot_group:
                 g = engine._slot_group[slot]
@@ -483,7 +507,7 @@ class _DecodeGraph:
         """Run the step once eagerly (every buffer then exists and the result is
         already right), then record the same launches."""
         with ops.stream_scope():
-            engine.model.forward(self.ctx)
+            engine._forward(self.ctx)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         stream = torch.cuda.Stream()
@@ -491,6 +515,6 @@ class _DecodeGraph:
         with torch.cuda.stream(stream):
             with torch.cuda.graph(graph, stream=stream):
                 with ops.stream_scope():
-                    self.logits = engine.model.forward(self.ctx)
+                    self.logits = engine._forward(self.ctx)
         torch.cuda.current_stream().wait_stream(stream)
         self.graph = graph

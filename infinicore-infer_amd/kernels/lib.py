@@ -37,6 +37,53 @@ class IcResidualNorm(_c.Structure):
     _fields_ = [("x", _P), ("ldx", _I), ("weight", _P), ("alpha", _F), ("sumsq_out", _P), ("n_parts", _I)]
 
 
+# ---- the native step function (see csrc/infinicore_infer_engine.h) -----------------------------------
+MAX_CACHE_GROUPS = 8
+
+
+class IcNorm(_c.Structure):
+    _fields_ = [("weight", _P), ("eps", _F)]
+
+
+class IcAttention(_c.Structure):
+    _fields_ = [("n_heads", _I), ("n_kv_heads", _I), ("head_dim", _I), ("window", _I), ("shared_kv", _I),
+                ("rot_dim", _I), ("max_positions", _I), ("softmax_scale", _F), ("cos", _P), ("sin", _P),
+                ("w_qkv", _P), ("w_o", _P)]
+
+
+class IcSwiGLU(_c.Structure):
+    _fields_ = [("intermediate", _I), ("w_gate_up", _P), ("w_down", _P)]
+
+
+class IcLayer(_c.Structure):
+    _fields_ = [("mixer_norm", IcNorm), ("attention", IcAttention), ("ffn_norm", IcNorm), ("ffn", IcSwiGLU),
+                ("residual_scale", _F)]
+
+
+class IcRunEntry(_c.Structure):
+    _fields_ = [("layer", _I), ("writes_cache", _I), ("group", _I), ("k_cache", _P), ("v_cache", _P)]
+
+
+class IcDecoderMeta(_c.Structure):
+    _fields_ = [("dtype", _I), ("hidden", _I), ("vocab", _I), ("page_size", _I), ("n_layers", _I), ("n_entries", _I),
+                ("n_groups", _I), ("compute_units", _I), ("embed_scale", _F), ("logit_scale", _F),
+                ("embed_table", _P), ("head_weight", _P), ("final_norm", IcNorm), ("final_norm_scaled", _P)]
+
+
+class IcStepBatch(_c.Structure):
+    _fields_ = [("n_tokens", _I), ("n_requests", _I), ("n_want", _I), ("n_decode_rows", _I), ("n_prefill_tiles", _I),
+                ("want_rows_identity", _I), ("decode_rows_identity", _I), ("max_position", _I), ("max_context", _I),
+                ("fixed_decode_splits", _I), ("tokens", _P), ("positions", _P), ("token_req", _P), ("want_rows", _P),
+                ("decode_rows", _P), ("prefill_tiles", _P), ("group_slots", _P * MAX_CACHE_GROUPS),
+                ("group_tables", _P * MAX_CACHE_GROUPS), ("group_table_stride", _I * MAX_CACHE_GROUPS)]
+
+
+class IcHostBatch(_c.Structure):
+    _fields_ = [("n_tokens", _I), ("n_requests", _I), ("tokens", _P), ("req_lens", _P), ("req_pos", _P),
+                ("want_count", _P), ("want", _P), ("tables", _P), ("table_len", _P), ("tile_rows", _I),
+                ("fixed_decode_splits", _I)]
+
+
 _RF = _c.POINTER(IcRowFactor)
 _RN = _c.POINTER(IcResidualNorm)
 
@@ -68,7 +115,19 @@ _SIGNATURES = {
     "ic_matmul_tune": [_P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _LL, _P, _LL, _I, _P],
     "ic_gemm_qkv_rope_tile_rows": [_I],
     "ic_gemm_nt_cfg": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
+    "ic_attn_decode_splits": [_I, _I, _I, _I, _I, _I],
+    "ic_decoder_create": [_c.POINTER(IcDecoderMeta), _c.POINTER(IcLayer), _c.POINTER(IcRunEntry)],
+    "ic_decoder_create_error": [],
+    "ic_decoder_destroy": [_P],
+    "ic_decoder_last_error": [_P],
+    "ic_decoder_workspace_bytes": [_P, _c.POINTER(IcStepBatch)],
+    "ic_decoder_forward": [_P, _c.POINTER(IcStepBatch), _P, _LL, _P, _LL, _P, _P],
+    "ic_decoder_step_ints": [_P, _c.POINTER(IcHostBatch)],
+    "ic_decoder_pack": [_P, _c.POINTER(IcHostBatch), _P, _P, _LL, _c.POINTER(IcStepBatch)],
+    "ic_decoder_step": [_P, _c.POINTER(IcHostBatch), _P, _P, _LL, _P, _LL, _P, _LL, _P, _c.POINTER(IcStepBatch), _P],
 }
+_RESTYPES = {"ic_decoder_create": _P, "ic_decoder_create_error": _c.c_char_p, "ic_decoder_destroy": None,
+             "ic_decoder_last_error": _c.c_char_p, "ic_decoder_workspace_bytes": _LL, "ic_decoder_step_ints": _LL}
 
 
 def get_lib():
@@ -87,7 +146,7 @@ def get_lib():
                 except AttributeError:
                     raise KernelError("kernel library %s lacks %s" % (path, name))
                 fn.argtypes = argtypes
-                fn.restype = _I
+                fn.restype = _RESTYPES.get(name, _I)
             _lib, _lib_path = lib, path
     return _lib
 

@@ -40,6 +40,11 @@ def _stream():
     return _scoped_stream if _scoped_stream is not None else torch.cuda.current_stream().cuda_stream
 
 
+def current_stream():
+    """The stream the kernels launch on (the scoped one inside ``stream_scope``)."""
+    return _stream()
+
+
 def _need(cond, what):
     if not cond:
         raise KernelError(what)
@@ -358,6 +363,11 @@ def _workspace(device):
     if ws is None:
         ws = _matmul_workspace[key] = torch.empty(MATMUL_WORKSPACE_BYTES, dtype=torch.uint8, device=device)
     return ws
+
+
+def library_workspace(device):
+    """The library products' scratch memory for the current stream on ``device``."""
+    return _workspace(device)
 
 
 class NoLibraryAlgorithm(KernelError):

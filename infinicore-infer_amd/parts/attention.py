@@ -77,6 +77,16 @@ class Attention(Mixer):
             self.w_qkv = torch.cat(mats, dim=0).contiguous() if len(mats) > 1 else mats[0]
         self.w_o = tensors[n + "o_proj.weight"]
 
+    def native_desc(self):
+        from ..kernels.lib import IcAttention
+        rot = getattr(self.pos_enc, "native_rotary", lambda: None)()
+        ws = (self.w_qkv, self.w_o)
+        if not (self._forward_is(Attention) and type(self)._attend is Attention._attend and rot is not None
+                and all(w is not None and w.is_cuda and w.dtype == self.runtime.dtype and w.is_contiguous() for w in ws)):
+            return None
+        return IcAttention(self.nh, self.nkvh, self.dh, self.window, int(self.shared_kv), rot[0], rot[1], self.scale,
+                           rot[2], rot[3], self.w_qkv.data_ptr(), self.w_o.data_ptr())
+
     # ---- forward ---------------------------------------------------------------------
     def forward(self, h, ctx, cache, tail=None):
         rt = self.runtime

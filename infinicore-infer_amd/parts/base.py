@@ -135,6 +135,17 @@ class Part:
     def sub_parts(self):
         return ()
 
+    def native_desc(self):
+        """What the native step function needs to run this part without Python: a description struct
+        of the kernel library's C interface (sizes, constants, weight addresses), or None when the
+        part has no native counterpart (then the whole model is stepped from Python).  A part that
+        overrides ``forward`` of a built-in part must not inherit its description."""
+        return None
+
+    def _forward_is(self, cls) -> bool:
+        """True when this object's forward is ``cls``'s own (no subclass changed what a step does)."""
+        return type(self).forward is cls.forward
+
     def position_limit(self):
         """Positions this part can take (a table's length), or None when it has no limit.  The
         engine refuses a step that would go beyond the smallest limit before it changes anything."""

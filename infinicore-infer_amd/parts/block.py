@@ -33,6 +33,18 @@ class PreNormResidualBlock(Block):
         d = norm.deferred()
         return None if d is None else ResidualTail(x, self.residual_scale, d[0], d[1])
 
+    def native_desc(self):
+        """The layer for the native step function, when it is this arrangement of parts that all have
+        a native description themselves (attention, SwiGLU, RMS norms)."""
+        from ..kernels.lib import IcAttention, IcLayer, IcNorm, IcSwiGLU
+        if not self._forward_is(PreNormResidualBlock):
+            return None
+        descs = [p.native_desc() for p in (self.mixer_norm, self.mixer, self.feed_forward_norm, self.feed_forward)]
+        if not (isinstance(descs[0], IcNorm) and isinstance(descs[1], IcAttention) and isinstance(descs[2], IcNorm)
+                and isinstance(descs[3], IcSwiGLU)):
+            return None
+        return IcLayer(descs[0], descs[1], descs[2], descs[3], self.residual_scale)
+
     def forward(self, x, pending, ctx, cache, successor=None):
         if isinstance(pending, DeferredRows):
             h = pending                               # the add is done; the mixer applies the row factors

@@ -39,6 +39,14 @@ class Embedding(Part):
     def forward(self, tokens, x):
         return ops.embed(tokens, self.table, x, self.scale)
 
+    def native_desc(self):
+        """(table address, scale) for the native step function."""
+        t = self.table
+        if not (self._forward_is(Embedding) and t is not None and t.is_cuda and t.dtype == self.runtime.dtype
+                and t.is_contiguous()):
+            return None
+        return (t.data_ptr(), self.scale)
+
 
 class _ScaledNorm:
     """(weight, eps) of a norm whose weight already carries the head's scale."""
@@ -87,6 +95,14 @@ class LMHead(Part):
         if key not in self._scaled_norms:
             self._scaled_norms[key] = _ScaledNorm((d[0] * self.logit_scale).contiguous(), d[1])
         return self._scaled_norms[key]
+
+    def native_desc(self):
+        """(weight address, logit scale) for the native step function."""
+        w = self.weight
+        if not (self._forward_is(LMHead) and w is not None and w.is_cuda and w.dtype == self.runtime.dtype
+                and w.is_contiguous()):
+            return None
+        return (w.data_ptr(), self.logit_scale)
 
     def forward(self, x, rows, final_norm, ctx):
         """Float32 logits [len(rows), vocab] of the residual rows ``rows``."""

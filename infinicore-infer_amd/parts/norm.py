@@ -2,6 +2,8 @@
 float32 residual stream (call sites src/models/jiuge/jiuge.cpp:198,246,262;
 eps = rms_norm_eps, scripts/jiuge.py:132; weights kept in float32,
 scripts/jiuge.py:146,209-215)."""
+import torch
+
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import Norm, register_part
@@ -31,3 +33,11 @@ class RMSNorm(Norm):
 
     def deferred(self):
         return (self.weight, self.eps)
+
+    def native_desc(self):
+        from ..kernels.lib import IcNorm
+        w = self.weight
+        if not (self._forward_is(RMSNorm) and w is not None and w.is_cuda and w.dtype == torch.float32
+                and w.is_contiguous()):
+            return None
+        return IcNorm(w.data_ptr(), self.eps)

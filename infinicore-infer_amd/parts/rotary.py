@@ -71,6 +71,13 @@ class Rotary(PositionEncoding):
     def position_limit(self):
         return self.max_positions
 
+    def native_rotary(self):
+        """(rot_dim, table rows, cos address, sin address) for the native step function."""
+        if type(self).rotate_and_store is not Rotary.rotate_and_store or \
+                type(self).project_rotate_store is not Rotary.project_rotate_store or not self.cos.is_cuda:
+            return None
+        return (self.rot_dim, self.max_positions, self.cos.data_ptr(), self.sin.data_ptr())
+
     def rotate_and_store(self, qkv, ctx, cache, n_heads, n_kv_heads, head_dim):
         if ctx.max_position >= self.max_positions:
             raise ValueError("position %d is beyond the rotary tables (%d)" % (ctx.max_position, self.max_positions))
@@ -104,6 +111,11 @@ class NoPositionEncoding(PositionEncoding):
 
     def __init__(self, name, runtime, **_):
         super().__init__(name, runtime)
+
+    def native_rotary(self):
+        if type(self).rotate_and_store is not NoPositionEncoding.rotate_and_store:
+            return None
+        return (0, 0, None, None)
 
     def rotate_and_store(self, qkv, ctx, cache, n_heads, n_kv_heads, head_dim):
         if n_kv_heads > 0:

@@ -46,6 +46,14 @@ class SwiGLU(FeedForward):
             self.w_gate_up = torch.cat([g, u], dim=0).contiguous()
         self.w_down = tensors[n + "down_proj.weight"]
 
+    def native_desc(self):
+        from ..kernels.lib import IcSwiGLU
+        ws = (self.w_gate_up, self.w_down)
+        if not (self._forward_is(SwiGLU)
+                and all(w is not None and w.is_cuda and w.dtype == self.runtime.dtype and w.is_contiguous() for w in ws)):
+            return None
+        return IcSwiGLU(self.intermediate_size, self.w_gate_up.data_ptr(), self.w_down.data_ptr())
+
     def forward(self, h, ctx, tail=None):
         rt = self.runtime
         T = h.shape[0]
