@@ -20,6 +20,7 @@ class Workspace:
         self.device = device
         self._bufs: Dict[tuple, torch.Tensor] = {}
         self._views: Dict[tuple, tuple] = {}     # (name, dtype) -> (shape, view): the view handed out last
+        self.frozen = False                      # True: buffers may not be regrown (recorded launches hold their addresses)
 
     def buffer(self, name: str, shape, dtype) -> torch.Tensor:
         key = (name, dtype)
@@ -32,6 +33,9 @@ class Workspace:
             n *= int(s)
         buf = self._bufs.get(key)
         if buf is None or buf.numel() < n:
+            if self.frozen:
+                raise RuntimeError("workspace buffer %r would have to grow from %d to %d elements, but recorded "
+                                   "steps hold its address" % (name, 0 if buf is None else buf.numel(), n))
             buf = torch.empty(max(n, 1), dtype=dtype, device=self.device)
             self._bufs[key] = buf
         view = buf[:n].view(*shape)

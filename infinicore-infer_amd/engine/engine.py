@@ -8,6 +8,7 @@ request.  Here the cache handle is a request id known to the cache manager;
 portions of prompts and single decoded tokens may be mixed and cut anywhere.
 """
 from dataclasses import dataclass, field
+from collections import OrderedDict
 from typing import Dict, List, Optional, Sequence
 
 import numpy as np
@@ -73,11 +74,12 @@ class _PinnedRing:
 class Engine:
     def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 64,
                  num_pages: Optional[int] = None, use_graphs: bool = True, graph_max_batch: int = 64,
-                 use_native: bool = True):
+                 use_native: bool = True, max_graphs: int = 32):
         """``max_tokens``: the most tokens live requests hold at any time, each
         request's count rounded up to whole pages; every group's pool is sized for it.
         ``use_native``: let one native call issue a step's kernels when every part of the model
-        has a native description (otherwise, and for other models, the parts' Python forward runs)."""
+        has a native description (otherwise, and for other models, the parts' Python forward runs).
+        ``max_graphs``: recorded decode steps kept at a time (the least recently used one goes first)."""
         self.model = model
         self.runtime: Runtime = model.runtime
         self.device = torch.device(self.runtime.device)
@@ -121,8 +123,12 @@ class Engine:
         # decode steps (one token per request, its logits wanted) replay a captured HIP graph
         self.use_graphs = bool(use_graphs) and all(p.graph_safe for p in model.all_parts())
         self.graph_max_batch = int(graph_max_batch)
-        self._graphs: Dict[tuple, "_DecodeGraph"] = {}
-        self.graph_replays = 0
+        self._graphs: "OrderedDict[tuple, _DecodeGraph]" = OrderedDict()
+        self.max_graphs = max(1, int(max_graphs))
+        self._graph_ws: Optional[Workspace] = None      # shared by all recorded steps of a natively stepped model
+        self.graph_steps = 0         # steps that took the recorded path (the recording one included)
+        self.graph_replays = 0       # of these, replays of an existing recording
+        self.graphs_evicted = 0
         # the step function in native code, when the model's parts all have a native description
         from .native import NativeDecoder
         self.native = NativeDecoder.try_build(self) if use_native else None
@@ -362,24 +368,57 @@ class Engine:
         (batch size, key split) into a HIP graph with those integers in a fixed device
         buffer, and replayed after one copy into that buffer."""
         R = len(entries)
-        ps = self.page_size
         bucket = _context_bucket(max(starts) + 1)
         key = (R, bucket)
         g = self._graphs.get(key)
         if g is None:
+            while len(self._graphs) >= self.max_graphs:          # the least recently used recording goes
+                self._graphs.popitem(last=False)
+                self.graphs_evicted += 1
             g = _DecodeGraph(self, R, bucket)
             self._graphs[key] = g
+        else:
+            self._graphs.move_to_end(key)
         g.fill(self, entries, starts)
         g.meta.copy_(g.host, non_blocking=True)
         g.copied.record()
         g.ctx.max_position = max(starts)
         g.ctx.req_pos = list(starts)
         g.ctx.req_ids = [e.req_id for e in entries]
+        self.graph_steps += 1
         if g.graph is None:
-            g.capture(self)
+            return g.capture(self)          # the first step of a shape runs eagerly (its result) and is recorded
         g.graph.replay()
         self.graph_replays += 1
         return g.logits
+
+    def _graph_workspace(self) -> Workspace:
+        """The workspace of recorded steps.  A natively stepped model needs one buffer whose size is
+        known beforehand, so all its recordings share one workspace made for the largest recorded
+        batch (only one runs at a time, on one stream): what recordings hold does not grow with their
+        number.  Otherwise every recording has a workspace of its own (its buffers are asked for by
+        name while it is recorded and must never move afterwards)."""
+        if self.native is None:
+            return Workspace(self.device)
+        if self._graph_ws is None:
+            ws = Workspace(self.device)
+            ws.buffer("native", (self.native.workspace_bytes_for_decode(self.graph_max_batch),), torch.uint8)
+            ws.buffer("logits", (self.graph_max_batch, self.model.spec.vocab_size), torch.float32)
+            ws.frozen = True
+            self._graph_ws = ws
+        return self._graph_ws
+
+    def graph_bytes(self) -> int:
+        """Device bytes held for recorded decode steps: workspaces and the steps' integer arrays."""
+        seen, total = set(), 0
+        for g in self._graphs.values():
+            total += g.meta.numel() * 4
+            if id(g.ctx.ws) not in seen:
+                seen.add(id(g.ctx.ws))
+                total += g.ctx.ws.bytes()
+        if self._graph_ws is not None and id(self._graph_ws) not in seen:
+            total += self._graph_ws.bytes()
+        return total
 
     # ---- library products ----------------------------------------------------------------------------
     def tune_library_products(self, token_counts: Sequence[int]) -> None:
@@ -455,8 +494,8 @@ class _DecodeGraph:
             return self.meta[self.off[n]:self.off[n] + sizes[n]]
 
         ctx = StepContext()
-        # a workspace of its own: the recorded launches hold its addresses, so it must never be regrown
-        ctx.T, ctx.R, ctx.page_size, ctx.ws = R, R, engine.page_size, Workspace(engine.device)
+        # the recorded launches hold the workspace's addresses, so it must never be regrown
+        ctx.T, ctx.R, ctx.page_size, ctx.ws = R, R, engine.page_size, engine._graph_workspace()
         ctx.tokens, ctx.positions, ctx.token_req = view("tokens"), view("positions"), view("token_req")
         ctx.state_slots = view("state_slots")
         ctx.want_rows, ctx.n_want, ctx.want_rows_identity = view("want_rows"), R, True
@@ -504,10 +543,11 @@ class _DecodeGraph:
         self.ctx.host_state_slots = slots
 
     def capture(self, engine):
-        """Run the step once eagerly (every buffer then exists and the result is
-        already right), then record the same launches."""
+        """Run the step once eagerly: that is the step's result, and every buffer then exists.  Then
+        record the same launches (recording executes nothing).  The step is therefore computed once,
+        also when it is recorded; a part that is ``graph_safe`` need not be idempotent."""
         with ops.stream_scope():
-            engine._forward(self.ctx)
+            logits = engine._forward(self.ctx)
         torch.cuda.synchronize()
         graph = torch.cuda.CUDAGraph()
         stream = torch.cuda.Stream()
@@ -517,4 +557,7 @@ class _DecodeGraph:
                 with ops.stream_scope():
                     self.logits = engine._forward(self.ctx)
         torch.cuda.current_stream().wait_stream(stream)
+        if self.logits is None or logits is None or self.logits.data_ptr() != logits.data_ptr():
+            raise RuntimeError("a recorded step must write its logits where the eager step did")
         self.graph = graph
+        return logits

@@ -69,6 +69,18 @@ class NativeDecoder:
                               % lib.ic_decoder_create_error().decode())
         return cls(handle, lib, model.spec.vocab_size, (layer_arr, entry_arr, meta, scaled_w))
 
+    def workspace_bytes_for_decode(self, n_requests: int) -> int:
+        """Workspace bytes that any step of up to ``n_requests`` single tokens needs (with the most key
+        splits the kernels take), for a workspace that recorded steps share and that must never grow."""
+        b = IcStepBatch()
+        b.n_tokens = b.n_requests = b.n_want = b.n_decode_rows = int(n_requests)
+        b.want_rows_identity = b.decode_rows_identity = 1
+        b.fixed_decode_splits = 64
+        need = self._bytes(self._h, ctypes.byref(b))
+        if need < 0:
+            raise KernelError("native step: no workspace size for %d single tokens" % n_requests)
+        return int(need)
+
     def forward(self, ctx, workspace_name: str = "native"):
         """Launch the step ``ctx`` describes; returns float32 logits [n_want, vocab] (a workspace view) or None."""
         b = self._batch

@@ -127,7 +127,7 @@ def test_decoding_twenty_requests_at_once(tmp_path_factory, name, dname, dtype, 
     ref = H.plain_logits(cfg, H.load_state_dict(folder), requests, dtype == torch.bfloat16)
     assert len(got) == n_req * (1 + n_dec)
     H.compare(got, ref, tol, "%s %s twenty requests" % (name, dname))
-    assert engine.graph_replays == n_dec
+    assert engine.graph_steps == n_dec and engine.graph_replays == n_dec - 1     # the first one records
     engine.cache.check_invariants()
 
 
@@ -177,7 +177,7 @@ def test_recorded_decode_steps_equal_eager_ones(tmp_path_factory, dname, dtype, 
     for i in range(6):                       # three requests
         ents = [StepEntry(k, [toks[20 + i + j]], [0]) for j, k in enumerate("pqr")]
         assert torch.equal(a.step(ents).clone(), b.step(ents).clone())
-    assert a.graph_replays == 18 and b.graph_replays == 0 and len(a._graphs) >= 3
+    assert a.graph_steps == 18 and b.graph_steps == 0 and len(a._graphs) >= 3 and a.graph_replays == 18 - len(a._graphs)
 
 
 @pytest.mark.parametrize("shape", ["2b", "1b", "8b"])
@@ -216,7 +216,7 @@ def test_recorded_steps_with_library_products_equal_eager_ones(tmp_path_factory,
                 for eng in (a, b):
                     eng.step([StepEntry("extra%d" % n_req, H.random_tokens(20011, 33, 5), [32])])
                     eng.free("extra%d" % n_req)
-    assert a.graph_replays == 10 and b.graph_replays == 0
+    assert a.graph_steps == 10 and a.graph_replays == 8 and b.graph_steps == 0
 
 
 def _random_configuration(seed):
@@ -351,4 +351,45 @@ def test_benchmark_shaped_layers(tmp_path_factory):
     for (rid, pos), row in got.items():
         err = float((row.double() - ref[rid][pos]).abs().max()) / scale
         assert err <= H.BF16_TOL, "request %s position %d differs by %.3g of the largest logit" % (rid, pos, err)
-    assert engine.graph_replays >= 9
+    assert engine.graph_steps >= 9
+
+
+@pytest.mark.parametrize("native", [True, False])
+def test_recorded_steps_hold_a_bounded_amount_of_memory(tmp_path_factory, native):
+    """Every batch size from 1 to 64 decodes once.  Recordings beyond ``max_graphs`` push out the least
+    recently used one; a natively stepped model's recordings share one workspace sized for the largest
+    batch, so the bytes they hold stay under a cap that does not depend on how many shapes were seen."""
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    cfg = H.CONFIGS["C"][0]
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "C")
+    eng = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=64 * 64, page_size=16, max_requests=64,
+                          max_graphs=12, use_native=native)
+    ids = ["g%d" % i for i in range(64)]
+    eng.step([StepEntry(r, H.random_tokens(cfg["vocab_size"], 3 + i % 9, i), []) for i, r in enumerate(ids)])
+    sizes = []
+    for n in range(1, 65):
+        out = eng.step([StepEntry(r, [1 + i], [0]) for i, r in enumerate(ids[:n])])
+        assert out.shape == (n, cfg["vocab_size"])
+        sizes.append(eng.graph_bytes())
+        assert len(eng._graphs) <= 12
+    assert eng.graph_steps == 64 and eng.graphs_evicted == 64 - 12
+    meta_bytes = 12 * 4 * (64 * (7 + cfg["max_position_embeddings"] // 16) + 64)
+    if native:
+        cap = eng.native.workspace_bytes_for_decode(64) + 64 * cfg["vocab_size"] * 4 + meta_bytes
+        assert max(sizes) <= cap, (max(sizes), cap)
+    else:
+        # a workspace per recording: bounded by max_graphs times the largest one
+        biggest = max(g.ctx.ws.bytes() + g.meta.numel() * 4 for g in eng._graphs.values())
+        assert max(sizes) <= 12 * biggest
+    assert sizes[-1] <= 1.05 * max(sizes[11:])            # no growth once the cap on recordings is reached
+    # a recording that was pushed out is made again when its shape comes back, with the right result
+    again = eng.step([StepEntry(r, [9], [0]) for r in ids[:2]]).clone()
+    ref = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=64 * 64, page_size=16, max_requests=64, use_graphs=False)
+    ref.step([StepEntry(r, H.random_tokens(cfg["vocab_size"], 3 + i % 9, i), []) for i, r in enumerate(ids[:2])])
+    for n in range(1, 65):
+        if n <= 2:
+            ref.step([StepEntry(r, [1 + i], [0]) for i, r in enumerate(ids[:min(n, 2)])])
+        else:
+            ref.step([StepEntry(r, [1 + i], [0]) for i, r in enumerate(ids[:2])])
+    want = ref.step([StepEntry(r, [9], [0]) for r in ids[:2]])      # other batches, other kernels: equal to rounding
+    assert float((again - want).abs().max()) <= H.BF16_TOL * float(want.abs().max())
