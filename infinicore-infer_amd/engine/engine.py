@@ -223,9 +223,8 @@ class Engine:
                     and all(len(e.tokens) == 1 and list(e.want) == [0] for e in entries)):
                 logits = self._graph_step(entries, starts)
             else:
-                ctx = self._build_context(entries, starts)
                 with ops.stream_scope():
-                    logits = self._forward(ctx)
+                    logits = self._eager_step(entries, starts)
         except BaseException:
             for e in entries:
                 if e.req_id in new_ids:
@@ -238,6 +237,19 @@ class Engine:
             self.cache.trim(e.req_id)
         self.steps_run += 1
         return logits
+
+    def _eager_step(self, entries, starts):
+        """A step that is not a replay: native code lays the batch out and launches it when the model
+        allows; otherwise the batch is packed here and the parts' forward runs."""
+        from ..parts import linear as _linear
+        if self.native is not None and not _linear.TUNE_LIBRARY:
+            try:
+                out = self.native.step(self, entries, starts)
+                self.native_steps += 1
+                return out
+            except ops.NoLibraryAlgorithm:
+                self.native = None        # see _forward; nothing of the half-issued step is kept
+        return self.model.forward(self._build_context(entries, starts))
 
     def _forward(self, ctx):
         """The model's forward for a packed step: issued by one native call when the model allows it

@@ -9,13 +9,15 @@ as before.  Both paths launch the same kernels with the same arguments, so their
 bit-equal (tested).
 """
 import ctypes
+from itertools import chain
 from typing import Optional
 
+import numpy as np
 import torch
 
 from ..kernels import ops
-from ..kernels.lib import (MAX_CACHE_GROUPS, IcDecoderMeta, IcLayer, IcNorm, IcRunEntry, IcStepBatch, KernelError,
-                           get_lib)
+from ..kernels.lib import (MAX_CACHE_GROUPS, IcDecoderMeta, IcHostBatch, IcLayer, IcNorm, IcRunEntry, IcStepBatch,
+                           KernelError, get_lib)
 
 
 class NativeDecoder:
@@ -81,6 +83,60 @@ class NativeDecoder:
             raise KernelError("native step: no workspace size for %d single tokens" % n_requests)
         return int(need)
 
+    def step(self, engine, entries, starts):
+        """A whole step from the entries themselves, the way the reference's inferBatch takes a batch
+        (tokens, req_lens, req_pos, one cache per request; include/infinicore_infer/models/jiuge.h:89-110):
+        native code lays the step's integers out in pinned memory, one copy takes them to the device,
+        one call launches the kernels.  Returns float32 logits [wanted, vocab] or None."""
+        lib, cache = self._lib, engine.cache
+        R, ng = len(entries), len(engine.groups)
+        lens = [len(e.tokens) for e in entries]
+        T = sum(lens)
+        tok = np.fromiter(chain.from_iterable(e.tokens for e in entries), dtype=np.int32, count=T)
+        req_lens = np.array(lens, dtype=np.int32)
+        req_pos = np.array(starts, dtype=np.int32)
+        want_count = np.array([len(e.want) for e in entries], dtype=np.int32)
+        n_want = int(want_count.sum())
+        want = np.fromiter(chain.from_iterable(e.want for e in entries), dtype=np.int32, count=n_want)
+        tables = [np.asarray(cache.block_table(e.req_id, g), dtype=np.int32) for g in range(ng) for e in entries]
+        ptrs = (ctypes.c_void_p * (ng * R))(*[t.ctypes.data for t in tables])
+        table_len = np.array([t.shape[0] for t in tables], dtype=np.int32)
+        hb = IcHostBatch(T, R, tok.ctypes.data, req_lens.ctypes.data, req_pos.ctypes.data, want_count.ctypes.data,
+                         want.ctypes.data, ctypes.cast(ptrs, ctypes.c_void_p), table_len.ctypes.data,
+                         engine._tile_rows, 0)
+        n = lib.ic_decoder_step_ints(self._h, ctypes.byref(hb))
+        if n < 0:
+            raise KernelError("native step: the batch is not valid (lengths, positions or block tables)")
+        host = engine._ring.get(n)
+        dev = engine._meta_dev
+        if dev is None or dev.numel() < n:
+            dev = engine._meta_dev = torch.empty(max(n, 4096), dtype=torch.int32, device=engine.device)
+        b = self._batch
+        st = lib.ic_decoder_pack(self._h, ctypes.byref(hb), host.data_ptr(), dev.data_ptr(), n, self._batch_ref)
+        if st:
+            raise KernelError("native step: laying out the batch failed (%d)" % st)
+        dev[:n].copy_(host[:n], non_blocking=True)
+        engine._ring.mark()
+        return self._launch(engine.ws, "native")
+
+    def _launch(self, workspace, workspace_name):
+        """Launch the step that ``self._batch`` describes."""
+        b = self._batch
+        need = self._bytes(self._h, self._batch_ref)
+        if need < 0:
+            raise KernelError("native step: the batch description is not valid")
+        ws = workspace.buffer(workspace_name, (need,), torch.uint8)
+        logits = workspace.buffer("logits", (b.n_want, self.vocab), torch.float32) if b.n_want else None
+        lib_ws = ops.library_workspace(ws.device)
+        st = self._forward(self._h, self._batch_ref, ws.data_ptr(), need, lib_ws.data_ptr(), ops.MATMUL_WORKSPACE_BYTES,
+                           logits.data_ptr() if logits is not None else None, ops.current_stream())
+        if st:
+            msg = self._lib.ic_decoder_last_error(self._h).decode()
+            if st == -4:
+                raise ops.NoLibraryAlgorithm("native step: " + msg)
+            raise KernelError("native step: " + msg)
+        return logits
+
     def forward(self, ctx, workspace_name: str = "native"):
         """Launch the step ``ctx`` describes; returns float32 logits [n_want, vocab] (a workspace view) or None."""
         b = self._batch
@@ -97,17 +153,4 @@ class NativeDecoder:
             b.group_slots[g] = slots.data_ptr()
             b.group_tables[g] = tables.data_ptr()
             b.group_table_stride[g] = tables.stride(0)
-        need = self._bytes(self._h, self._batch_ref)
-        if need < 0:
-            raise KernelError("native step: the batch description is not valid")
-        ws = ctx.ws.buffer(workspace_name, (need,), torch.uint8)
-        logits = ctx.ws.buffer("logits", (ctx.n_want, self.vocab), torch.float32) if ctx.n_want else None
-        lib_ws = ops.library_workspace(ws.device)
-        st = self._forward(self._h, self._batch_ref, ws.data_ptr(), need, lib_ws.data_ptr(), ops.MATMUL_WORKSPACE_BYTES,
-                           logits.data_ptr() if logits is not None else None, ops.current_stream())
-        if st:
-            msg = self._lib.ic_decoder_last_error(self._h).decode()
-            if st == -4:
-                raise ops.NoLibraryAlgorithm("native step: " + msg)
-            raise KernelError("native step: " + msg)
-        return logits
+        return self._launch(ctx.ws, workspace_name)

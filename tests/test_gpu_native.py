@@ -98,3 +98,75 @@ def test_models_with_parts_of_their_own_are_stepped_from_python(tmp_path_factory
     plain = build_model(spec, Runtime(torch.bfloat16, "cuda:0"))
     init_random_weights(plain, seed=1)
     assert Engine(plain, max_tokens=128).native is not None
+
+
+def test_the_c_step_function_through_ctypes(tmp_path_factory):
+    """ic_decoder_step as a C caller would use it, without the engine's Python around it: host arrays in the
+    shape of inferBatch (tokens, req_lens, req_pos, a block table per request), a pinned staging buffer,
+    device memory for the integers and the workspace.  Two steps (prompts of three requests; then single
+    tokens of two of them beside a portion of the third) against an engine that is fed the same."""
+    import ctypes
+    import numpy as np
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    from infinicore_infer_amd.kernels.lib import IcHostBatch, IcStepBatch, get_lib
+    cfg = H.CONFIGS["C"][0]
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "C")
+    eng = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=1024, page_size=16, max_requests=4)
+    ref = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=1024, page_size=16, max_requests=4, use_native=False)
+    lib, dec = get_lib(), eng.native._h
+    dev = torch.device("cuda:0")
+    prompts = [H.random_tokens(cfg["vocab_size"], n, 40 + i) for i, n in enumerate([150, 9, 70])]
+    # the caller's own bookkeeping: pages 0.. handed out in order, 16 tokens a page
+    tables = [[], [], []]
+    next_page = [0]
+
+    def grow(r, length):
+        while len(tables[r]) * 16 < length:
+            tables[r].append(next_page[0])
+            next_page[0] += 1
+
+    staging = torch.empty(1 << 16, dtype=torch.int32, pin_memory=True)
+    ints = torch.empty(1 << 16, dtype=torch.int32, device=dev)
+    work = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    lib_ws = torch.empty(64 << 20, dtype=torch.uint8, device=dev)
+    stream = torch.cuda.current_stream().cuda_stream
+
+    def c_step(reqs, toks, pos, want):
+        lens = [len(t) for t in toks]
+        for r, t, p in zip(reqs, toks, pos):
+            grow(r, p + len(t))
+        tok = np.array([x for t in toks for x in t], dtype=np.int32)
+        req_lens, req_pos = np.array(lens, dtype=np.int32), np.array(pos, dtype=np.int32)
+        want_count = np.array([len(w) for w in want], dtype=np.int32)
+        want_flat = np.array([x for w in want for x in w], dtype=np.int32)
+        tabs = [np.array(tables[r], dtype=np.int32) for r in reqs]
+        ptrs = (ctypes.c_void_p * len(reqs))(*[t.ctypes.data for t in tabs])
+        tlen = np.array([len(t) for t in tabs], dtype=np.int32)
+        hb = IcHostBatch(len(tok), len(reqs), tok.ctypes.data, req_lens.ctypes.data, req_pos.ctypes.data,
+                         want_count.ctypes.data, want_flat.ctypes.data, ctypes.cast(ptrs, ctypes.c_void_p),
+                         tlen.ctypes.data, lib.ic_attn_prefill_tile_rows(), 0)
+        n = lib.ic_decoder_step_ints(dec, ctypes.byref(hb))
+        assert 0 < n <= staging.numel()
+        logits = torch.empty(int(want_count.sum()), cfg["vocab_size"], dtype=torch.float32, device=dev)
+        laid = IcStepBatch()
+        st = lib.ic_decoder_step(dec, ctypes.byref(hb), staging.data_ptr(), ints.data_ptr(), n, work.data_ptr(),
+                                 work.numel(), lib_ws.data_ptr(), lib_ws.numel(), logits.data_ptr(),
+                                 ctypes.byref(laid), stream)
+        assert st == 0, lib.ic_decoder_last_error(dec).decode()
+        torch.cuda.synchronize()
+        assert lib.ic_decoder_workspace_bytes(dec, ctypes.byref(laid)) <= work.numel()
+        return logits, laid
+
+    got, laid = c_step([0, 1, 2], [prompts[0], prompts[1], prompts[2][:40]], [0, 0, 0], [[0, 149], [8], []])
+    assert (laid.n_tokens, laid.n_requests, laid.n_want, laid.n_decode_rows) == (199, 3, 3, 0)
+    want = ref.step([StepEntry("a", prompts[0], [0, 149]), StepEntry("b", prompts[1], [8]),
+                     StepEntry("c", prompts[2][:40], [])])
+    # the reference engine hands out pages in the same order, so even the cache slots agree; the logits must
+    assert torch.equal(got, want)
+    got, laid = c_step([1, 2, 0], [[5], prompts[2][40:], [7]], [9, 40, 150], [[0], [0, 29], [0]])
+    assert (laid.n_decode_rows, laid.n_prefill_tiles, laid.want_rows_identity) == (2, 1, 0)
+    want = ref.step([StepEntry("b", [5], [0]), StepEntry("c", prompts[2][40:], [0, 29]), StepEntry("a", [7], [0])])
+    assert torch.equal(got, want)
+    # a batch that does not add up is refused before anything is launched
+    bad = IcHostBatch(5, 1, 0, 0, 0, 0, 0, 0, 0, 128, 0)
+    assert lib.ic_decoder_step_ints(dec, ctypes.byref(bad)) == -1

@@ -209,17 +209,17 @@ def test_a_failure_inside_the_step_puts_the_cache_back(tmp_path_factory):
     toks = H.random_tokens(256, 60, 2)
     engine.step([StepEntry("x", toks[:20], [])])
     free, slots = engine.cache.free_pages(0), engine.cache.slots.n_free
-    real = engine._forward
+    real = engine._eager_step
 
-    def broken(ctx):
-        real(ctx)                                     # the step's kernels run, then the failure
+    def broken(entries, starts):
+        real(entries, starts)                         # the step's kernels run, then the failure
         raise ops.KernelError("forced failure")
-    engine._forward = broken
+    engine._eager_step = broken
     try:
         with pytest.raises(ops.KernelError):
             engine.step([StepEntry("x", toks[20:50], [0]), StepEntry("n", toks[:33], [0])])
     finally:
-        engine._forward = real
+        engine._eager_step = real
     assert engine.length("x") == 20 and not engine.has_request("n")
     assert engine.cache.free_pages(0) == free and engine.cache.slots.n_free == slots
     engine.cache.check_invariants()
