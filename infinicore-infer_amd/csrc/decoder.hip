@@ -18,6 +18,7 @@
 namespace {
 
 constexpr int kFewRows = 16;        // up to here the few-row products beat the library
+constexpr int kMidRows = 64;        // up to here the sliced product beats it for results as wide as the model
 constexpr int kMaxSumsqParts = 256; // column blocks of sums of squares a product takes as row factors
 
 thread_local std::string g_create_error;
@@ -28,7 +29,7 @@ inline int dtype_size(int dtype) { return dtype == IC_BF16 ? 2 : 4; }
 struct Workspace {
     // byte offsets into the caller's workspace
     size_t residual, normed, qkv, attn_out, mixer_out, ffn_out, mixer_tail, mixer_sumsq, ffn_tail, ffn_sumsq, gate_up, act,
-        part_acc, part_ml, head_in, total;
+        part_acc, part_ml, head_in, tail_parts, total;
 };
 
 // Rows whose norm is half done: values = x * w, sums of squares per column block; the row factor
@@ -93,6 +94,13 @@ struct IcDecoder {
         w.part_acc = take(acc * 4);
         w.part_ml = take(ml * 4);
         w.head_in = take((size_t)b.n_want * d * ds);
+        size_t slices = 0;           // the O and down products of 17..64 rows as slices over K
+        if (meta.dtype == IC_BF16 && T > kFewRows && T <= kMidRows)
+            for (const IcLayer& l : layers) {
+                slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, l.attention.n_heads * l.attention.head_dim));
+                slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, l.ffn.intermediate));
+            }
+        w.tail_parts = take(slices * T * d * 4);
         w.total = o;
         return w;
     }
@@ -107,6 +115,22 @@ struct IcDecoder {
         }
         if (rows) return IC_ERR_ARG;      // half-normed rows exist only where the few-row product runs
         return ic_matmul(a, meta.dtype, w, out, out_dtype, M, N, K, lda, K, N, alpha, lib_ws, lib_ws_bytes, stream);
+    }
+
+    // 17..64 rows into the residual stream: x += alpha * (a w^T), out = rmsnorm(x) * weight, through the sliced
+    // product when it pays.  Returns 1 when done, 0 when the caller has to take the other way, < 0 on a fault.
+    int tail_in_slices(const void* a, int K, const void* w, float* parts, float* x, float alpha, const float* weight, float eps,
+                       void* out, int T, hipStream_t stream, int* status) const {
+        const int d = meta.hidden;
+        *status = IC_OK;
+        if (meta.dtype != IC_BF16 || T <= kFewRows || T > kMidRows || d % 4 || !ic_gemm_splitk_supported(T, d, K, K, K) ||
+            !ic_gemm_splitk_pays(T, d, K))
+            return 0;
+        const int slices = ic_gemm_splitk_slices(d, K);
+        *status = ic_gemm_splitk(a, w, parts, T, d, K, K, K, slices, stream);
+        if (*status) return -1;
+        *status = ic_splitk_add_rmsnorm(parts, slices, T, x, alpha, weight, out, d, eps, stream);
+        return *status ? -1 : 1;
     }
 
     int forward(const IcStepBatch& b, void* workspace, long long workspace_bytes, void* lib_ws, long long lib_ws_bytes,
@@ -133,7 +157,7 @@ struct IcDecoder {
         if (st) return fail(st, "the embedding gather", -1);
 
         // what the residual stream still owes when a layer starts
-        enum { NONE, BRANCH, DEFERRED } owed = NONE;
+        enum { NONE, BRANCH, DEFERRED, NORMED } owed = NONE;      // NORMED: the add and the whole norm are done, `normed` holds the rows
         const void* branch = nullptr;
         float branch_alpha = 0.f;
         Deferred def;
@@ -153,7 +177,8 @@ struct IcDecoder {
             // ---- norm before the mixer -------------------------------------------------------------
             const Deferred* h_def = nullptr;
             if (owed == DEFERRED) h_def = &def;
-            else if (owed == NONE) {
+            else if (owed == NORMED) {
+            } else if (owed == NONE) {
                 st = ic_rmsnorm(x, nullptr, L.mixer_norm.weight, normed, dt, T, d, L.mixer_norm.eps, 1.0f, stream);
                 if (st) return fail(st, "the norm before attention", i);
             } else {
@@ -218,7 +243,11 @@ struct IcDecoder {
             // ---- O projection, residual add, norm before the feed-forward --------------------------------
             Deferred mid;
             const Deferred* g_def = nullptr;
-            if (can_split_norm) {
+            const int sliced = tail_in_slices(attn_out, ow, A.w_o, (float*)(base + ws.tail_parts), x, L.residual_scale, L.ffn_norm.weight,
+                                              L.ffn_norm.eps, normed, T, stream, &st);
+            if (sliced < 0) return fail(st, "the O product in slices with residual add and norm", i);
+            if (sliced) {
+            } else if (can_split_norm) {
                 IcResidualNorm tail{x, d, L.ffn_norm.weight, L.residual_scale, (float*)(base + ws.mixer_sumsq), parts};
                 st = ic_gemm_nt(attn_out, IC_BF16, A.w_o, IC_BF16, base + ws.mixer_tail, IC_BF16, T, d, ow, ow, ow, d, 1.0f, 2, nullptr,
                                 &tail, stream);
@@ -248,7 +277,12 @@ struct IcDecoder {
                 st = ic_swiglu(base + ws.gate_up, act, dt, T, di, stream);
                 if (st) return fail(st, "SwiGLU", i);
             }
-            if (succ && can_split_norm) {
+            const int sliced_down = !succ ? 0 : tail_in_slices(act, di, L.ffn.w_down, (float*)(base + ws.tail_parts), x, L.residual_scale,
+                                                               succ_weight, succ->eps, normed, T, stream, &st);
+            if (sliced_down < 0) return fail(st, "the down product in slices with residual add and norm", i);
+            if (sliced_down) {
+                owed = NORMED;
+            } else if (succ && can_split_norm) {
                 IcResidualNorm tail{x, d, succ_weight, L.residual_scale, (float*)(base + ws.ffn_sumsq), parts};
                 st = ic_gemm_nt(act, IC_BF16, L.ffn.w_down, IC_BF16, base + ws.ffn_tail, IC_BF16, T, d, di, di, di, d, 1.0f, 2, nullptr,
                                 &tail, stream);
@@ -266,6 +300,11 @@ struct IcDecoder {
 
         // ---- final norm and head, on the wanted rows only -----------------------------------------------------
         if (b.n_want == 0) return IC_OK;
+        if (owed == NORMED) {        // every row in order, the final norm (with the logit scale in its weight) applied
+            st = linear(normed, d, meta.head_weight, logits, IC_F32, T, meta.vocab, d, 1.0f, nullptr, lib_ws, lib_ws_bytes, stream);
+            if (st) return fail(st, "the head product", -1);
+            return IC_OK;
+        }
         if (owed == DEFERRED) {      // every row in order, the final norm half done: its row factors go into the product
             st = linear(def.values, d, meta.head_weight, logits, IC_F32, T, meta.vocab, d, 1.0f, &def, lib_ws, lib_ws_bytes, stream);
             if (st) return fail(st, "the head product", -1);

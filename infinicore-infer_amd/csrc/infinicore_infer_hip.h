@@ -78,6 +78,17 @@ int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int ld
 // For tuning and tests: used weight rows per tile of ic_gemm_qkv_rope (16, 8 or 4; 0: chosen from the number of heads).
 int ic_gemm_qkv_rope_tile_rows(int rows);
 
+// ---- gemm_splitk.hip ----------------------------------------------------------------------------------
+// Products of 1..64 rows (bfloat16) as float32 slices over K, P[s, m, n] = A[m, K_s] . W[n, K_s], and the kernel
+// that sums the slices, adds them to the residual stream and applies the norm that follows.  For the O and down
+// projections of 17..64 rows, where it beats the library's product (ic_gemm_splitk_pays says when).
+int ic_gemm_splitk_supported(int M, int N, int K, int lda, int ldw);
+int ic_gemm_splitk_slices(int N, int K);      // how many slices to use (never an empty one)
+int ic_gemm_splitk_pays(int M, int N, int K);
+int ic_gemm_splitk(const void* A, const void* W, float* P, int M, int N, int K, int lda, int ldw, int n_slices, hipStream_t stream);
+// P [S, M, d]: x += alpha * (the product, rounded to bfloat16); out = rmsnorm(x) * w.
+int ic_splitk_add_rmsnorm(const float* P, int n_slices, int M, float* x, float alpha, const float* w, void* out, int d, float eps, hipStream_t stream);
+
 // ---- matmul_library.hip ------------------------------------------------------------------------------
 // The library (hipBLASLt) matrix product for many rows: C[M, N] = alpha * A[M, K] W[N, K]^T, bfloat16 operands with a
 // bfloat16 or float32 result, or all float32 (true float32).  Descriptors and the algorithm are kept per shape.

@@ -481,3 +481,45 @@ def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads
                                      sin.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), n_heads, n_kv_heads,
                                      head_dim, page_size, ctypes.byref(rf) if rf else None, _stream()), "gemm_qkv_rope")
     return qkv
+
+
+# ---- products of 17..64 rows as slices over K, and what follows them -------------------------------------------
+def gemm_splitk_supported(a, w) -> bool:
+    return bool(a.dtype == torch.bfloat16 and w.dtype == torch.bfloat16 and a.dim() == 2 and w.dim() == 2
+                and a.stride(1) == 1 and w.stride(1) == 1 and a.shape[1] == w.shape[1]
+                and get_lib().ic_gemm_splitk_supported(a.shape[0], w.shape[0], a.shape[1], a.stride(0), w.stride(0)))
+
+
+def gemm_splitk_pays(m: int, n: int, k: int) -> bool:
+    """True when the sliced product beats the library's for an m x n x k product (17..64 rows, enough blocks)."""
+    return bool(get_lib().ic_gemm_splitk_pays(int(m), int(n), int(k)))
+
+
+def gemm_splitk_slices(n: int, k: int) -> int:
+    return int(get_lib().ic_gemm_splitk_slices(int(n), int(k)))
+
+
+def gemm_splitk(a, w, parts, n_slices=None):
+    """parts[s, m, n] (float32) = a[m, K_s] . w[n, K_s] for the slices K_s of K; 1..64 rows, bfloat16 operands.
+    ``parts`` must hold n_slices * M * N floats; returns its [n_slices, M, N] view."""
+    _dev(a, w, parts)
+    M, K = a.shape
+    N = w.shape[0]
+    _need(gemm_splitk_supported(a, w), "gemm_splitk: at most 64 bfloat16 rows, K a multiple of 8, rows 16-byte aligned")
+    S = int(n_slices) if n_slices else gemm_splitk_slices(N, K)
+    _need(parts.dtype == torch.float32 and parts.is_contiguous() and parts.numel() >= S * M * N, "gemm_splitk: parts too small")
+    check(get_lib().ic_gemm_splitk(a.data_ptr(), w.data_ptr(), parts.data_ptr(), M, N, K, a.stride(0), w.stride(0), S, _stream()),
+          "gemm_splitk")
+    return parts.view(-1)[:S * M * N].view(S, M, N)
+
+
+def splitk_add_rmsnorm(parts, x, alpha: float, weight, out, eps: float):
+    """x += alpha * (the product given as slices parts [S, M, d], rounded to bfloat16); out = rmsnorm(x) * weight."""
+    _dev(parts, x, weight, out)
+    S, M, d = parts.shape
+    _need(parts.dtype == torch.float32 and parts.is_contiguous() and x.dtype == torch.float32 and x.is_contiguous()
+          and tuple(x.shape) == (M, d) and weight.dtype == torch.float32 and weight.numel() == d and weight.is_contiguous()
+          and out.dtype == torch.bfloat16 and out.is_contiguous() and tuple(out.shape) == (M, d), "splitk_add_rmsnorm: layout")
+    check(get_lib().ic_splitk_add_rmsnorm(parts.data_ptr(), S, M, x.data_ptr(), float(alpha), weight.data_ptr(), out.data_ptr(),
+                                          d, float(eps), _stream()), "splitk_add_rmsnorm")
+    return out

@@ -47,9 +47,11 @@ class DeferredRows:
     """Rows whose norm is half done.  ``values[r]`` is x[r] * w (the norm's weight is applied, its
     row factor is not); ``sumsq[b, r]`` are sums of x[r]^2 over column blocks b.  The true row is
     values[r] * rsqrt(sumsq[:, r].sum() / width + eps).  The row factor commutes with a projection,
-    so a part that takes such rows (``accepts_deferred``) applies it to its first product's result."""
+    so a part that takes such rows (``accepts_deferred``) applies it to its first product's result.
+    ``sumsq`` None: the producer has applied the whole norm already and ``values`` are the normed rows
+    (nothing is owed); consumers then treat them as a plain tensor."""
     values: torch.Tensor
-    sumsq: torch.Tensor                # float32 [n_parts, 16]
+    sumsq: Optional[torch.Tensor]      # float32 [n_parts, 16], or None
     width: int
     eps: float
 
@@ -62,10 +64,12 @@ class DeferredRows:
         return self.values.dtype
 
     def row_factor(self):
-        return (self.sumsq, self.width, self.eps)
+        return None if self.sumsq is None else (self.sumsq, self.width, self.eps)
 
     def materialize(self):
         """The normed rows as a plain tensor (slow path for parts of a product that cannot take factors)."""
+        if self.sumsq is None:
+            return self.values
         T = self.values.shape[0]
         f = torch.rsqrt(self.sumsq.sum(0)[:T, None] / self.width + self.eps)
         return (self.values.to(torch.float32) * f).to(self.values.dtype)

@@ -17,6 +17,7 @@ torch.backends.cuda.matmul.allow_tf32 = False
 torch.backends.cudnn.allow_tf32 = False
 
 FEW_ROWS = 16          # up to here the package's own kernel beats the library on MI355X
+MID_ROWS = 64          # up to here the sliced product beats it for results as wide as the model (O, down)
 TUNE_LIBRARY = False   # while True, every library product times the library's algorithms for its shape first
 TUNE_FLUSH = None      # while tuning: a tensor larger than the caches, overwritten before every timed launch
 _tuned = set()
@@ -72,7 +73,18 @@ def linear_tail(x, w, tail, ws, name: str, impl: str = "auto"):
     epilogue: returns ``DeferredRows`` for that norm, or None when this step cannot be done so
     (many rows, float32, a width beyond the kernel's) and the caller computes the plain product."""
     M, N = x.shape[0], w.shape[0]
-    if tail is None or not own_kernel_applies(M, x.dtype, w.dtype, torch.bfloat16, impl):
+    if tail is None:
+        return None
+    if (impl == "auto" and FEW_ROWS < M <= MID_ROWS and tuple(tail.x.shape) == (M, N) and N % 4 == 0
+            and ops.gemm_splitk_supported(x, w) and ops.gemm_splitk_pays(M, N, w.shape[1])):
+        # 17..64 rows into the residual stream: the product as slices over K; the kernel that sums them does
+        # the add and the whole norm, so the rows handed on owe nothing
+        slices = ops.gemm_splitk_slices(N, w.shape[1])
+        parts = ops.gemm_splitk(x, w, ws.buffer("tail_parts", (slices * M * N,), torch.float32), slices)
+        y = ws.buffer(name + "_values", (M, N), torch.bfloat16)
+        ops.splitk_add_rmsnorm(parts, tail.x, tail.alpha, tail.weight, y, tail.eps)
+        return DeferredRows(y, None, N, tail.eps)
+    if not own_kernel_applies(M, x.dtype, w.dtype, torch.bfloat16, impl):
         return None
     parts = ops.residual_parts(N)
     if parts > ops.MAX_SUMSQ_PARTS or tuple(tail.x.shape) != (M, N):

@@ -602,3 +602,55 @@ def test_gemm_qkv_rope_with_row_factors():
     _close(qkv[:, :nh * dh], ref[:, :nh * dh], torch.bfloat16)
     _close(kc, kc2, torch.bfloat16)
     _close(vc, vc2, torch.bfloat16)
+
+
+# ---------------------------------------------------------------------------
+@pytest.mark.parametrize("M,N,K,S", [(1, 64, 128, 1), (17, 2304, 2304, 0), (33, 200, 344, 1), (64, 2304, 5760, 0), (48, 1000, 1096, 2),
+                                      (64, 331, 8, 1), (20, 4096, 8192, 0), (64, 136, 520, 1), (31, 777, 1160, 3)])
+def test_gemm_in_slices_and_the_add_norm_that_sums_them(M, N, K, S):
+    """The product of 1..64 rows as float32 slices over K (sizes that are no multiple of the block's 64 columns
+    or of its chunk of 128 k; slices of unequal length), against float64; then the kernel that sums the slices,
+    rounds to bfloat16, adds to the residual stream and applies the norm, against the same steps in float64."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(M * 1000 + N + K)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
+    w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
+    assert ops.gemm_splitk_supported(a, w)
+    slices = S or ops.gemm_splitk_slices(N, K)
+    parts = torch.full((slices * M * N + 64,), float("nan"), device=DEV)
+    p = ops.gemm_splitk(a, w, parts, slices)
+    assert p.shape == (slices, M, N)
+    assert bool(torch.isnan(parts[slices * M * N:]).all())            # nothing written beyond the slices
+    want = a.double().cpu() @ w.double().cpu().t()
+    _close(p.double().sum(0), want, torch.float32, factor=4)
+    if S == 0:                                                        # the library's own choice: slices it says are not empty
+        assert 1 <= slices <= 64
+    if N % 4:
+        return
+    x = torch.randn(M, N, generator=g).to(DEV)
+    weight = (1 + 0.1 * torch.randn(N, generator=g)).to(DEV)
+    out = torch.empty(M, N, dtype=torch.bfloat16, device=DEV)
+    x_before = x.double().cpu()
+    ops.splitk_add_rmsnorm(p, x, 0.37, weight, out, 1e-5)
+    t = p[0].cpu().clone()                                            # the slices summed in float32 in the kernel's order, so
+    for i in range(1, slices):                                        # that the rounding to bfloat16 (the product as it would
+        t += p[i].cpu()                                               # be stored) falls the same way
+    y = t.to(torch.bfloat16).double()
+    x_want = x_before + 0.37 * y
+    _close(x, x_want, torch.float32, factor=4)
+    _close(out, P.plain_rmsnorm(x_want, weight.double().cpu(), 1e-5), torch.bfloat16)
+
+
+def test_gemm_in_slices_refuses_what_it_does_not_take():
+    ops = _ops()
+    a = torch.zeros(65, 64, dtype=torch.bfloat16, device=DEV)
+    w = torch.zeros(64, 64, dtype=torch.bfloat16, device=DEV)
+    assert not ops.gemm_splitk_supported(a, w)                        # more than 64 rows
+    assert not ops.gemm_splitk_supported(a[:8, :60], w[:, :60])       # K no multiple of 8
+    assert not ops.gemm_splitk_supported(a[:8].float(), w.float())
+    with pytest.raises(ops.KernelError):
+        ops.gemm_splitk(a, w, torch.empty(65 * 64, device=DEV), 1)
+    with pytest.raises(ops.KernelError):                              # a slice would be empty: 1 chunk, 2 slices
+        ops.gemm_splitk(a[:8], w, torch.empty(2 * 8 * 64, device=DEV), 2)
+    assert not ops.gemm_splitk_pays(16, 2304, 2304) and not ops.gemm_splitk_pays(65, 2304, 2304)
+    assert not ops.gemm_splitk_pays(32, 200, 344)                     # too few blocks for the chip
