@@ -180,6 +180,47 @@ class CacheManager:
             e.first_live[g] = min(e.first_live[g], len(table))
         e.length = length
 
+    def rename(self, old_id, new_id) -> None:
+        """Hand everything ``old_id`` holds (pages, state slot, length) to ``new_id``: a new request
+        takes over a finished one's cache to go on from a common prefix."""
+        if new_id in self.requests:
+            raise CacheError("request %r is already admitted" % (new_id,))
+        e = self.requests.pop(old_id)
+        self._admissions += 1
+        e.serial = self._admissions               # a new life: recorded steps must not take its block table for the old one
+        self.requests[new_id] = e
+
+    def fork(self, src_id, dst_id, n_tokens: Optional[int] = None):
+        """Admit ``dst_id`` with pages of its own for the first ``n_tokens`` tokens of ``src_id`` (all of
+        them by default).  Returns (state slot of dst, [(group, src page, dst page), ...]): the pages whose
+        contents the caller has to copy.  All or nothing: with too few pages or no slot nothing changes.
+        The reference copies a cache the same way, duplicateKVCache (src/models/jiuge/jiuge_kv_cache.cpp:25-47)."""
+        src = self.requests[src_id]
+        n = src.length if n_tokens is None else int(n_tokens)
+        if not (0 <= n <= src.length):
+            raise CacheError("fork: request %r holds %d tokens, %d asked" % (src_id, src.length, n))
+        if dst_id in self.requests:
+            raise CacheError("request %r is already admitted" % (dst_id,))
+        if self.slots.n_free == 0:
+            raise OutOfPages("no free state slot (max_requests = %d)" % self.max_requests)
+        n_pages = self._pages_for(n)
+        live = [[j for j in range(min(n_pages, len(t))) if t[j] >= 0] for t in src.tables]
+        for g, idx in enumerate(live):
+            if len(idx) > self.pools[g].n_free:
+                raise OutOfPages("fork needs %d pages of group %d, %d free" % (len(idx), g, self.pools[g].n_free))
+        slot = self.admit(dst_id)
+        dst = self.requests[dst_id]
+        pairs = []
+        for g, idx in enumerate(live):
+            table = [-1] * n_pages                # pages the source gave back (behind a window) stay given back
+            for j in idx:
+                table[j] = self.pools[g].alloc()
+                pairs.append((g, src.tables[g][j], table[j]))
+            dst.tables[g] = table
+            dst.first_live[g] = min(src.first_live[g], n_pages)
+        dst.length = n
+        return slot, pairs
+
     def trim(self, req_id) -> int:
         """Give back the pages of window groups that no later token can read.
         Call after the step that appended has been launched.  Returns the count."""

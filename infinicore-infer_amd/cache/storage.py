@@ -46,6 +46,19 @@ class CacheStorage:
             kv = self._kv_views[slot] = (self.group_planes[g][i, 0], self.group_planes[g][i, 1])
         return kv
 
+    def copy_pages(self, group: int, src_pages: Sequence[int], dst_pages: Sequence[int]) -> None:
+        """Copy whole pages inside a group: every cache slot of the group, keys and values."""
+        if not src_pages:
+            return
+        from ..kernels import ops
+        planes = self.group_planes[group]
+        idx = torch.tensor([list(src_pages), list(dst_pages)], dtype=torch.int32).to(self.device)
+        ops.copy_pages(planes, idx[0].contiguous(), idx[1].contiguous())
+
+    def copy_state(self, src_slot: int, dst_slot: int) -> None:
+        for t in self.state.values():
+            t[dst_slot].copy_(t[src_slot])
+
     def zero_state(self, state_slot: int) -> None:
         for t in self.state.values():
             t[state_slot].zero_()

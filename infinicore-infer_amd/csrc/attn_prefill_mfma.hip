@@ -50,16 +50,18 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                          int n_tiles, int nh, int nkvh, int page_shift, float scale_log2e, int window) {
     constexpr int NC = DH / 16;           // 16-wide chunks of the head dimension
     constexpr int ND = DH / 32;           // 32-row tiles of O^T
-    constexpr int KS = DH + kPfPad;       // row stride of Ks and Vs (elements)
+    constexpr int KS = DH + kPfPad;       // row stride of Ks (elements): 16-byte reads of 8 consecutive rows cover all banks
+    constexpr int VS = DH + 2 * kPfPad;   // row stride of Vs: the transposing 8-byte reads touch 4 rows at once, which must
+                                          // fall into different banks (a stride of 32 bytes mod 128; with KS two rows share one)
     constexpr int kPfThreads = kPfWaveThreads * GROUPS;
     constexpr int STEP = kPfKeys * GROUPS;                 // keys staged per step
     constexpr int NL = STEP * (DH / 8) / kPfThreads;       // 16-byte loads per thread per plane and step
-    constexpr int KT = kPfKeys * KS, VT = KT;              // elements of one group's K and V tile
+    constexpr int KT = kPfKeys * KS, VT = kPfKeys * VS;    // elements of one group's K and V tile
     constexpr int MERGE_F = 2 + ND * 16;                   // floats a lane hands over at the end
     static_assert(GROUPS == 1 || sizeof(uint16_t) * GROUPS * (KT + VT) >= sizeof(float) * 256 * MERGE_F, "merge buffer fits in the tiles");
     __shared__ __attribute__((aligned(16))) uint16_t tilebuf[GROUPS * (KT + VT)];
     uint16_t* const Ks_all = tilebuf;                      // [group][key][KS]
-    uint16_t* const Vs_all = tilebuf + GROUPS * KT;     // [group][key][KS]
+    uint16_t* const Vs_all = tilebuf + GROUPS * KT;     // [group][key][VS]
 
     __shared__ int pages[kPfMaxPages];
 
@@ -160,9 +162,8 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         for (int i = 0; i < NL; ++i) {
             const int idx = tid + i * kPfThreads;
             const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
-            const int at = (key / kPfKeys) * KT + (key % kPfKeys) * KS + oct * 8;
-            *reinterpret_cast<uint4*>(&Ks_all[at]) = kreg[i];
-            *reinterpret_cast<uint4*>(&Vs_all[at]) = vreg[i];
+            *reinterpret_cast<uint4*>(&Ks_all[(key / kPfKeys) * KT + (key % kPfKeys) * KS + oct * 8]) = kreg[i];
+            *reinterpret_cast<uint4*>(&Vs_all[(key / kPfKeys) * VT + (key % kPfKeys) * VS + oct * 8]) = vreg[i];
         }
     };
 
@@ -246,10 +247,10 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             for (int dt = 0; dt < ND; ++dt) {
                 // this lane's chunk: key 16 kc + 4 half + (l % 16) / 4 (and 8 keys on), dims 32 dt + 16 (l / 16 % 2) + 4 (l % 4) ..+3;
                 // what comes back is dim 32 dt + lq of keys 16 kc + 4 half + e (and 8 keys on), e = 0..3
-                const uint16_t* vp = &Vs[(16 * kc + 4 * half + ((lane & 15) >> 2)) * KS + 32 * dt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)];
+                const uint16_t* vp = &Vs[(16 * kc + 4 * half + ((lane & 15) >> 2)) * VS + 32 * dt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)];
                 Frag8 a;
                 a.h[0] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)vp));
-                a.h[1] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)(vp + 8 * KS)));
+                a.h[1] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)(vp + 8 * VS)));
                 oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b, oacc[dt], 0, 0, 0);
             }
         }

@@ -283,3 +283,29 @@ IC_EXPORT int ic_swiglu(const void* gate_up, void* out, int dtype, int T, int di
         return IC_ERR_UNSUPPORTED;
     return ic_launch_status();
 }
+
+
+// ---------------------------------------------------------------------------
+// Whole pages copied inside the planes of a cache group: for every plane p (a cache slot's keys or
+// values) planes[p][dst[i]] = planes[p][src[i]].  Grid (pairs, planes); 16 bytes a thread and turn.
+// ---------------------------------------------------------------------------
+__global__ void __launch_bounds__(256)
+copy_pages_kernel(uint4* __restrict__ planes, const int* __restrict__ src, const int* __restrict__ dst,
+                  long long plane_vecs, long long page_vecs) {
+    const uint4* from = planes + (size_t)blockIdx.y * plane_vecs + (size_t)src[blockIdx.x] * page_vecs;
+    uint4* to = planes + (size_t)blockIdx.y * plane_vecs + (size_t)dst[blockIdx.x] * page_vecs;
+    for (long long i = threadIdx.x; i < page_vecs; i += 256) to[i] = from[i];
+}
+
+// planes: n_planes planes of n_pages pages of page_bytes bytes each, one after the other.  src, dst: device int32 [n_pairs],
+// page ids < n_pages; a page must not be both a source and a destination of one call.
+IC_EXPORT int ic_copy_pages(void* planes, int n_planes, long long n_pages, long long page_bytes, const int* src, const int* dst,
+                            int n_pairs, hipStream_t stream) {
+    if (n_pairs <= 0 || n_planes <= 0) return IC_OK;
+    if (!planes || !src || !dst || n_pages <= 0 || page_bytes <= 0 || page_bytes % 16 || ((uintptr_t)planes & 15) ||
+        n_planes > 65535)
+        return IC_ERR_ARG;
+    hipLaunchKernelGGL(copy_pages_kernel, dim3(n_pairs, n_planes), dim3(256), 0, stream, (uint4*)planes, src, dst,
+                       n_pages * (page_bytes / 16), page_bytes / 16);
+    return ic_launch_status();
+}

@@ -28,6 +28,10 @@ int ic_residual_add(float* x, const void* y, int y_dtype, float alpha, long long
 // out[t, j] = up * silu(gate), gate = gate_up[t, j], up = gate_up[t, di + j].
 int ic_swiglu(const void* gate_up, void* out, int dtype, int T, int di, hipStream_t stream);
 
+// Whole cache pages copied inside a group's planes (n_planes planes of n_pages pages of page_bytes bytes, contiguous):
+// planes[p][dst[i]] = planes[p][src[i]] for every plane p.  src, dst: device int32 [n_pairs]; no page both read and written.
+int ic_copy_pages(void* planes, int n_planes, long long n_pages, long long page_bytes, const int* src, const int* dst, int n_pairs, hipStream_t stream);
+
 // ---- rope_kv.hip ------------------------------------------------------------------------------
 // Rotary on the q and k heads of qkv[T, row_stride] (pairs (j, j + rot/2)), k and v written to cache slot slots[t].
 int ic_rope_kv_write(void* qkv, int dtype, const int* positions, const float* cos_t, const float* sin_t, void* kcache, void* vcache, const int* slots, int T, int row_stride, int nh, int nkvh, int dh, int rot, int page_size, hipStream_t stream);

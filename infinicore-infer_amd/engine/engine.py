@@ -113,6 +113,7 @@ class Engine:
             if need.kind == "state":
                 self.storage.add_state(slot, self.max_requests, need.state_shape, need.state_dtype)
         self._slot_group = {s: g for g, spec in enumerate(self.groups) for s in spec.slots}
+        self.has_state = bool(self.storage.state)      # some mixer keeps fixed-size state per request
 
         self.ws = Workspace(self.device)
         self._ring = _PinnedRing()
@@ -166,6 +167,25 @@ class Engine:
 
     def length(self, req_id) -> int:
         return self.cache.length(req_id)
+
+    def fork(self, src_id, dst_id, n_tokens: Optional[int] = None) -> None:
+        """A new request ``dst_id`` that holds a copy of the first ``n_tokens`` cached tokens of
+        ``src_id`` (all by default) in pages of its own; both go on independently.  What the
+        reference's duplicateKVCache does for its slabs (src/models/jiuge/jiuge_kv_cache.cpp:25-47).
+        Fixed-size state of ``src_id`` is copied as it is now, so with such state only a full copy
+        (``n_tokens`` None or the whole length) is meaningful."""
+        slot, pairs = self.cache.fork(src_id, dst_id, n_tokens)
+        for g in range(len(self.groups)):
+            mine = [(s, d) for gg, s, d in pairs if gg == g]
+            self.storage.copy_pages(g, [s for s, _ in mine], [d for _, d in mine])
+        if self.storage.state:
+            self.storage.copy_state(self.cache.state_slot(src_id), slot)
+
+    def adopt(self, old_id, new_id, n_tokens: int) -> None:
+        """``new_id`` takes over the cache of ``old_id`` cut down to its first ``n_tokens`` tokens: a new
+        request goes on from the prefix it shares with a finished one (scripts/kvcache_pool.py:18-42)."""
+        self.cache.rename(old_id, new_id)
+        self.cache.truncate(new_id, n_tokens)
 
     # ---- the step ----------------------------------------------------------------------------
     def step(self, entries: Sequence[StepEntry]):

@@ -13,6 +13,11 @@ there is no token budget and memory is committed per whole-context slab
   * every step takes all running requests that decode (one token each) first,
     then prompt portions of at most ``chunk_size`` tokens until
     ``max_batch_tokens`` are spent;
+  * with ``prefix_cache`` a finished request's cache is kept, with the tokens it holds, until its
+    pages are needed; a new request takes over the kept cache that shares the longest prefix with
+    its prompt and starts at min(shared, prompt length - 1), the reference pool's rule
+    (scripts/kvcache_pool.py:18-42,58-76).  Kept caches are given up, oldest first, before any
+    running request is preempted;
   * when pages run out for a decode token, the most recently admitted running
     request is preempted: its pages and slot are given back and it returns to
     the FRONT of the waiting queue with prompt + generated tokens to be
@@ -24,7 +29,7 @@ The scheduler only needs ``engine.cache`` (a CacheManager), ``engine.step``,
 ``engine.sample``, ``engine.add_request`` and ``engine.free``, so its decisions
 are tested on the CPU with a stand-in engine.
 """
-from collections import deque
+from collections import OrderedDict, deque
 from dataclasses import dataclass, field
 from typing import Deque, Dict, List, Optional, Tuple
 
@@ -48,7 +53,7 @@ class _Running:
 
 class Scheduler:
     def __init__(self, engine, max_batch_tokens: int = 2048, chunk_size: int = 512,
-                 max_running: Optional[int] = None):
+                 max_running: Optional[int] = None, prefix_cache: bool = False):
         if max_batch_tokens < 1 or chunk_size < 1:
             raise ValueError("max_batch_tokens and chunk_size must be positive")
         self.engine = engine
@@ -63,6 +68,14 @@ class Scheduler:
         self.n_preempted = 0
         self.n_steps = 0
         self.last_plan: List[Tuple[object, int, int]] = []     # (id, first position, tokens) of the last step
+        # Kept caches of finished requests: only where every key stays available (no window group gives
+        # pages back) and no fixed-size state exists (a state cannot be cut back to a prefix).
+        self.prefix_cache = (bool(prefix_cache) and all(g.kind == "full" for g in self.cache.groups)
+                             and not getattr(engine, "has_state", False))
+        self.idle: "OrderedDict[object, List[int]]" = OrderedDict()    # kept cache id -> the tokens it holds, oldest first
+        self._idle_serial = 0
+        self.n_prefix_hits = 0
+        self.prefix_tokens_reused = 0
 
     # ---- queueing -----------------------------------------------------------------
     def add(self, task: InferTask) -> None:
@@ -86,7 +99,14 @@ class Scheduler:
     # ---- internals --------------------------------------------------------------------
     def _finish(self, r: _Running, reason: str) -> None:
         r.task.finish_reason = reason
-        self.engine.free(r.task.id)
+        held = self.cache.length(r.task.id) if self.cache.has_request(r.task.id) else 0
+        if self.prefix_cache and reason in ("stop", "length") and held > 0:
+            self._idle_serial += 1
+            kept = ("kept", self._idle_serial)
+            self.engine.adopt(r.task.id, kept, held)          # the cache stays, under a name of its own
+            self.idle[kept] = (list(r.task.prompt) + list(r.task.generated))[:held]
+        else:
+            self.engine.free(r.task.id)
         if r in self.running:
             self.running.remove(r)
         self.finished.append(r.task)
@@ -99,6 +119,34 @@ class Scheduler:
         r.cursor = 0
         self.waiting.appendleft(r)
         self.n_preempted += 1
+
+    def _evict_idle(self, keep=None) -> bool:
+        """Give up the oldest kept cache (not ``keep``); False when there is none."""
+        for kept in self.idle:
+            if kept != keep:
+                del self.idle[kept]
+                self.engine.free(kept)
+                return True
+        return False
+
+    def release_idle(self) -> None:
+        """Give up every kept cache."""
+        while self._evict_idle():
+            pass
+
+    def _best_prefix(self, feed: List[int]):
+        """(kept cache id, tokens to reuse) with the longest common prefix, by the reference's rule
+        min(shared, len - 1) so that at least one token is left to compute; (None, 0) without a match."""
+        best, best_n = None, 0
+        for kept, toks in self.idle.items():
+            n = 0
+            for a, b in zip(feed, toks):
+                if a != b:
+                    break
+                n += 1
+            if n > best_n:
+                best, best_n = kept, n
+        return best, min(best_n, len(feed) - 1)
 
     def _pages_for_new(self, n_tokens: int) -> List[int]:
         ps = self.cache.page_size
@@ -126,6 +174,8 @@ class Scheduler:
                     plan.append((r, 1))
                     budget -= 1
                     break
+                if self._evict_idle():                # kept caches of finished requests go before anyone running
+                    continue
                 victim = max(self.running, key=lambda x: x.order)
                 planned = [p for p in plan if p[0] is victim]
                 if planned:                      # a younger request already has its page this step: take it back
@@ -146,6 +196,8 @@ class Scheduler:
                 break
             n = min(self.chunk_size, len(r.feed) - r.cursor, budget)
             need = self.cache.pages_needed(r.task.id, n)
+            while not self._fits(need, reserved) and self._evict_idle():
+                pass
             if not self._fits(need, reserved):
                 continue
             reserved = [a + b for a, b in zip(reserved, need)]
@@ -153,20 +205,35 @@ class Scheduler:
             budget -= n
 
         # 3. admissions, first come first served
-        while self.waiting and budget >= 1 and len(self.running) < self.max_running \
-                and self.cache.slots.n_free > 0:
+        while self.waiting and budget >= 1 and len(self.running) < self.max_running:
             r = self.waiting[0]
             if self.cache.max_positions is not None and len(r.feed) > self.cache.max_positions:
                 self.waiting.popleft()
                 r.task.finish_reason = "length"
                 self.finished.append(r.task)
                 continue
-            n = min(self.chunk_size, len(r.feed), budget)
-            need = self._pages_for_new(n)
+            kept, shared = self._best_prefix(r.feed) if self.idle else (None, 0)
+            if kept is None or shared < 1:
+                kept, shared = None, 0
+                if self.cache.slots.n_free == 0 and not self._evict_idle():
+                    break
+            n = min(self.chunk_size, len(r.feed) - shared, budget)
+            ps = self.cache.page_size
+            have = (shared + ps - 1) // ps                       # pages the kept prefix brings along
+            need = [max(0, (shared + n + ps - 1) // ps - have)] * len(self.cache.groups)
+            while not self._fits(need, reserved) and self._evict_idle(keep=kept):
+                pass
             if not self._fits(need, reserved):
                 break
             self.waiting.popleft()
-            self.engine.add_request(r.task.id)
+            if kept is not None:
+                del self.idle[kept]
+                self.engine.adopt(kept, r.task.id, shared)       # go on from the shared prefix
+                r.cursor = shared
+                self.n_prefix_hits += 1
+                self.prefix_tokens_reused += shared
+            else:
+                self.engine.add_request(r.task.id)
             self._admitted += 1
             r.order = self._admitted
             self.running.append(r)
@@ -175,6 +242,9 @@ class Scheduler:
             budget -= n
 
         # nothing can move although requests run: make room by preempting the youngest
+        if not plan and self.idle and (self.running or self.waiting):
+            self.release_idle()                       # kept caches stood in the way
+            return self.plan()
         if not plan and self.running:
             victim = max(self.running, key=lambda x: x.order)
             if len(self.running) == 1:

@@ -93,6 +93,7 @@ _SIGNATURES = {
     "ic_add_rmsnorm": [_P, _P, _I, _F, _P, _P, _I, _I, _I, _F, _P],
     "ic_residual_add": [_P, _P, _I, _F, _LL, _P],
     "ic_swiglu": [_P, _P, _I, _I, _I, _P],
+    "ic_copy_pages": [_P, _I, _LL, _LL, _P, _P, _I, _P],
     "ic_rope_kv_write": [_P, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P],
     "ic_attn_generic": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _P, _I, _I, _I, _I, _I, _F, _I, _P],
     "ic_attn_decode_supported": [_I, _I],

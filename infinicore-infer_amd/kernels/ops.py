@@ -125,6 +125,19 @@ def swiglu(gate_up, out):
     return out
 
 
+def copy_pages(planes, src, dst):
+    """planes[..., dst[i], :, :, :] = planes[..., src[i], :, :, :] for a cache group's planes
+    [slots, 2, pages, kv_heads, page_size, head_dim] (contiguous); src, dst: int32 page ids on the device."""
+    _dev(planes, src, dst)
+    _i32(src, "src")
+    _i32(dst, "dst")
+    _need(planes.dim() == 6 and planes.is_contiguous() and src.numel() == dst.numel(), "copy_pages: layout")
+    n_pages = planes.shape[2]
+    page_bytes = planes.shape[3] * planes.shape[4] * planes.shape[5] * planes.element_size()
+    check(get_lib().ic_copy_pages(planes.data_ptr(), planes.shape[0] * planes.shape[1], n_pages, page_bytes,
+                                  src.data_ptr(), dst.data_ptr(), src.numel(), _stream()), "copy_pages")
+
+
 def rope_kv_write(qkv, positions, cos, sin, kcache, vcache, slots, n_heads, n_kv_heads, head_dim,
                   rot_dim, page_size):
     """Rotate the q heads of qkv[T, H] in place; rotate the k heads and copy the

@@ -34,10 +34,13 @@ _DTYPES = {"bfloat16": torch.bfloat16, "bf16": torch.bfloat16, "float32": torch.
 
 class MiniCPMForCausalLM:
     def __init__(self, model_dir_path, device="cuda:0", ndev=1, max_tokens=None, dtype=None,
-                 cache_tokens: Optional[int] = None, page_size: int = 64, max_requests: int = 64):
+                 cache_tokens: Optional[int] = None, page_size: int = 64, max_requests: int = 64,
+                 prefix_cache: bool = False):
         """``max_tokens`` caps the context length as in the reference
         (scripts/jiuge.py:128-130); ``cache_tokens`` sizes the page pool (default:
-        four full contexts); ``dtype`` None takes the checkpoint's torch_dtype."""
+        four full contexts); ``dtype`` None takes the checkpoint's torch_dtype; ``prefix_cache``
+        keeps finished requests' caches so that later prompts go on from a shared prefix, as the
+        reference's server pool does (scripts/kvcache_pool.py)."""
         if ndev != 1:
             raise ValueError("this engine runs on one GPU (ndev=%r)" % (ndev,))
         print("Loading model weights to host...")
@@ -49,6 +52,8 @@ class MiniCPMForCausalLM:
                                       max_tokens=cache_tokens or 4 * ctx, page_size=page_size,
                                       max_requests=max_requests)
         self.tokenizer = self._load_tokenizer(model_dir_path)
+        self.prefix_cache = bool(prefix_cache)
+        self._scheduler = None                  # kept between calls when finished requests' caches are kept
         print(f"Time used: {time.time() - t0:.3f}s")
 
     @staticmethod
@@ -73,6 +78,14 @@ class MiniCPMForCausalLM:
 
     def drop_kv_cache(self, kv_cache):
         kv_cache.drop(self)
+
+    def duplicate_kv_cache(self, kv_cache, seq_len: Optional[int] = None):
+        """A second cache holding a copy of the first ``seq_len`` tokens of ``kv_cache``
+        (duplicateKVCache, include/infinicore_infer/models/jiuge.h:66-69)."""
+        new = KVCache(self)
+        self.engine.fork(kv_cache.data(), new.data(), seq_len)
+        new.tokens = list(kv_cache.tokens[:self.engine.length(new.data())])
+        return new
 
     def batch_infer_one_round(self, tasks: List[InferTask]):
         """One step over the tasks' pending tokens; one sampled token per task
@@ -139,7 +152,14 @@ class MiniCPMForCausalLM:
     def _run_requests(self, prompts, max_new_tokens, topp_, topk_, temperature_, seed, max_batch_tokens,
                       chunk_size, on_step=None):
         """The one generation loop: every request is a task of the scheduler."""
-        sched = Scheduler(self.engine, max_batch_tokens=max_batch_tokens, chunk_size=chunk_size)
+        if self.prefix_cache:                   # one scheduler for the model's life: it holds the kept caches
+            if self._scheduler is None:
+                self._scheduler = Scheduler(self.engine, max_batch_tokens=max_batch_tokens, chunk_size=chunk_size,
+                                            prefix_cache=True)
+            sched = self._scheduler
+            sched.max_batch_tokens, sched.chunk_size = max_batch_tokens, chunk_size
+        else:
+            sched = Scheduler(self.engine, max_batch_tokens=max_batch_tokens, chunk_size=chunk_size)
         tasks = [InferTask("g%d" % i, list(p), self.max_context_len(), temperature_, topk_, topp_,
                            self.eos_token_id, seed=seed, max_new_tokens=max_new_tokens)
                  for i, p in enumerate(prompts)]
@@ -171,6 +191,9 @@ class MiniCPMForCausalLM:
         return math.exp(nll / total)
 
     def destroy_model_instance(self):
+        if self._scheduler is not None:
+            self._scheduler.release_idle()
+        self._scheduler = None
         self.engine = None
         torch.cuda.empty_cache()
         print("Model destroyed")
@@ -184,7 +207,7 @@ USAGE = ("Usage: python -m infinicore_infer_amd.minicpm [--amd] <path/to/model_d
          "options: [--device cuda:0] [--dtype bfloat16|float32] [--max-tokens N] [--prompt TEXT | --prompt-ids 1,2,3 ... | "
          "--prompt-len N [--num-prompts K]] [--max-new-tokens N] [--temperature T] [--top-k K] [--top-p P] [--seed S] "
          "[--page-size 16|32|64] [--num-pages N | --cache-tokens N] [--max-batch-tokens N] [--chunk-size N] "
-         "[--weights-seed S] [--weights-std X] [--weights-norm-std X]")
+         "[--prefix-cache] [--weights-seed S] [--weights-std X] [--weights-norm-std X]")
 
 _OTHER_DEVICES = ("--cpu", "--nvidia", "--cambricon", "--ascend", "--metax", "--moore", "--iluvatar")
 
@@ -228,6 +251,8 @@ def _parse(argv):
     ap.add_argument("--cache-tokens", type=int, default=None, help="tokens the page pool holds (default: four contexts)")
     ap.add_argument("--max-batch-tokens", type=int, default=2048, help="tokens per step over all requests")
     ap.add_argument("--chunk-size", type=int, default=512, help="largest portion of a prompt per step")
+    ap.add_argument("--prefix-cache", action="store_true",
+                    help="keep finished requests' caches; later prompts go on from a shared prefix")
     args = ap.parse_args(argv)
     if (model_path is None) == (not args.random_weights):
         print("give a model folder, or --random-weights --config <config.json>")
@@ -263,7 +288,7 @@ def test(argv=None):
         cache_tokens = args.num_pages * args.page_size
     model = MiniCPMForCausalLM(model_path, args.device, ndev, max_tokens=args.max_tokens,
                                dtype=_DTYPES[args.dtype] if args.dtype else None,
-                               cache_tokens=cache_tokens, page_size=args.page_size)
+                               cache_tokens=cache_tokens, page_size=args.page_size, prefix_cache=args.prefix_cache)
     if args.prompt_ids:
         prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     elif args.prompt_len:

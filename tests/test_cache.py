@@ -94,6 +94,24 @@ def test_random_orders_conserve_pages(seed):
                                       [list(t) for t in m.requests[r].tables])
                 else:
                     m.trim(r)
+        elif op < 0.86 and live and m.can_admit():          # a copy of a request's first tokens in pages of its own
+            r = rng.choice(live)
+            n += 1
+            try:
+                _, pairs = m.fork(r, n, rng.randint(0, m.length(r)))
+                live.append(n)
+                assert len({(g, d) for g, _, d in pairs}) == len(pairs)
+            except OutOfPages:
+                assert not m.has_request(n)
+        elif op < 0.9 and live:                              # a request's cache under a new name, cut back
+            r = live.pop(rng.randrange(len(live)))
+            n += 1
+            if any(g.kind == "window" for g in m.groups):
+                m.rename(r, n)
+            else:
+                m.rename(r, n)
+                m.truncate(n, rng.randint(0, m.length(n)))
+            live.append(n)
         elif live:
             r = live.pop(rng.randrange(len(live)))
             m.release(r)
@@ -121,4 +139,26 @@ def test_truncate_gives_back_exactly_what_the_appends_took():
     assert m.block_table("a", 0) == [] and m.free_pages(0) == 8
     with pytest.raises(Exception):
         m.truncate("a", 5)                      # it cannot grow a request
+    m.check_invariants()
+
+
+def test_fork_copies_the_first_tokens_into_pages_of_its_own():
+    m = CacheManager([FULL, WIN], [16, 16], 16, max_requests=3, max_positions=400)
+    m.admit("a")
+    m.append("a", 100)
+    m.trim("a")                                   # the window group gave its first pages back
+    slot, pairs = m.fork("a", "b", 70)
+    assert m.length("b") == 70 and slot == m.state_slot("b") != m.state_slot("a")
+    full = [(s, d) for g, s, d in pairs if g == 0]
+    assert [s for s, _ in full] == m.block_table("a", 0)[:5] and [d for _, d in full] == m.block_table("b", 0)
+    assert not set(m.block_table("b", 0)) & set(m.block_table("a", 0))
+    win_b = m.block_table("b", 1)
+    assert len(win_b) == 5 and [p < 0 for p in win_b] == [p < 0 for p in m.block_table("a", 1)[:5]]
+    m.check_invariants()
+    with pytest.raises(Exception):
+        m.fork("a", "c", 101)                      # more than the source holds
+    with pytest.raises(OutOfPages):
+        m.fork("a", "c", 100) or m.fork("a", "d", 100)      # the second one finds no state slot
+    m.release("a")
+    m.append("b", 20)                              # the copy goes on by itself
     m.check_invariants()

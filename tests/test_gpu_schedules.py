@@ -352,3 +352,66 @@ def test_kernels_round_to_bfloat16_to_nearest_even_and_keep_nan():
     xo = torch.empty(1, 16, dtype=torch.float32, device=dev)
     ops.embed(torch.zeros(1, dtype=torch.int32, device=dev), table, xo, 1.0)
     assert torch.equal(xo.view(torch.int32), table.float().view(torch.int32))
+
+
+# ---- a copy of a request's cache, and going on from a shared prefix ------------------------------------------------------
+@pytest.mark.parametrize("dname,dtype,tol", DTYPES)
+@pytest.mark.parametrize("name", ["B", "C"])
+def test_forked_requests_go_on_independently(tmp_path_factory, name, dname, dtype, tol):
+    """Engine.fork copies the first tokens of a request into pages of its own (the reference's
+    duplicateKVCache).  The copy, fed other tokens, and the original, fed its own, both match the plain
+    implementation; a full copy fed the same token gives the very same logits as the original."""
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    cfg = H.CONFIGS[name][0]
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), name)
+    eng = Engine.from_dir(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4)
+    a = H.random_tokens(cfg["vocab_size"], 90, 1)
+    b = a[:53] + H.random_tokens(cfg["vocab_size"], 30, 2)          # shares 53 tokens: the cut lies inside a page
+    eng.step([StepEntry("a", a[:70], [])])
+    eng.fork("a", "b", 53)
+    assert eng.length("b") == 53 and not set(eng.cache.block_table("a", 0)) & set(eng.cache.block_table("b", 0))
+    eng.cache.check_invariants()
+    got = {}
+    la = eng.step([StepEntry("a", a[70:], list(range(20))), StepEntry("b", b[53:], list(range(30)))]).float().cpu()
+    for i in range(20):
+        got[("a", 70 + i)] = la[i].clone()
+    for i in range(30):
+        got[("b", 53 + i)] = la[20 + i].clone()
+    ref = H.plain_logits(cfg, H.load_state_dict(folder), {"a": a, "b": b}, dtype == torch.bfloat16)
+    H.compare(got, ref, tol, "%s %s fork" % (name, dname))
+    eng.fork("a", "c")                                              # all of it
+    l1 = eng.step([StepEntry("a", [7], [0])]).clone()
+    l2 = eng.step([StepEntry("c", [7], [0])]).clone()
+    assert torch.equal(l1, l2)
+    for r in "abc":
+        eng.free(r)
+    eng.cache.check_invariants()
+    assert eng.cache.free_pages(0) == eng.num_pages
+
+
+@pytest.mark.parametrize("name", ["A", "C"])
+def test_prefix_cache_through_the_entry_point(tmp_path, name):
+    """With the prefix cache on, a second prompt that starts like a finished request goes on from the shared
+    tokens: fewer tokens are computed, the generated tokens are the plain implementation's (float32)."""
+    from plain_model import plain_generate
+    from infinicore_infer_amd.minicpm import MiniCPMForCausalLM
+    cfg = H.CONFIGS[name][0]
+    folder = H.make_model_dir(tmp_path, name, seed=8)
+    sd = H.load_state_dict(folder)
+    cfg_no_eos = dict(cfg)
+    model = MiniCPMForCausalLM(folder, dtype=torch.float32, cache_tokens=512, page_size=16, prefix_cache=True)
+    model.eos_token_id = []                                          # the lengths are what the test fixes
+    system = H.random_tokens(cfg["vocab_size"], 37, 3)
+    p1, p2 = system + [5, 6, 7], system + [9, 8]
+    out1 = model.generate_batch([p1], 6)[0]
+    assert out1 == plain_generate(cfg_no_eos, sd, p1, 6)
+    steps_before = model.engine.steps_run
+    out2 = model.generate_batch([p2], 6, chunk_size=4)[0]            # the rest of the prompt is 2 tokens: one portion
+    assert out2 == plain_generate(cfg_no_eos, sd, p2, 6)
+    sched = model.last_scheduler
+    assert sched.n_prefix_hits == 1 and sched.prefix_tokens_reused == 37
+    assert model.engine.steps_run - steps_before == 6               # one step for the 2 new prompt tokens, five to decode
+    # kept caches are given back with the model
+    model._scheduler.release_idle()
+    model.engine.cache.check_invariants()
+    assert model.engine.cache.free_pages(0) == model.engine.num_pages

@@ -34,6 +34,11 @@ class FakeEngine:
             self.cache.release(rid)
             del self.history[rid]
 
+    def adopt(self, old, new, n_tokens):
+        self.cache.rename(old, new)
+        self.cache.truncate(new, n_tokens)
+        self.history[new] = self.history.pop(old)[:n_tokens]
+
     def step(self, entries):
         assert len({e.req_id for e in entries}) == len(entries)
         rows = []
@@ -223,3 +228,74 @@ def test_command_line_arguments():
                 ["/m", "--device", "cpu"]):
         with pytest.raises(SystemExit):
             _parse(bad)
+
+
+def test_a_new_request_goes_on_from_the_prefix_it_shares_with_a_finished_one():
+    """The reference's pool keeps finished requests' caches and hands a new task the one with the longest
+    common prefix, starting at min(shared, len - 1) (scripts/kvcache_pool.py:18-42,58-76)."""
+    eng = FakeEngine(num_pages=32, max_requests=4)
+    s = Scheduler(eng, max_batch_tokens=64, chunk_size=64, prefix_cache=True)
+    system = list(range(20, 60))                                  # 40 tokens both prompts start with
+    a = _task("a", system + [1, 2, 3], 5)
+    s.add(a)
+    s.run()
+    assert a.generated == _expected(system + [1, 2, 3], 5)
+    assert len(s.idle) == 1 and eng.cache.free_pages() < 32      # its cache is kept
+    kept_tokens = list(s.idle.values())[0]
+    assert kept_tokens == (system + [1, 2, 3] + a.generated)[:47]     # the last token's keys were never computed
+    fed_before = sum(n for step in eng.steps for _, n in step)
+    b = _task("b", system + [7, 8, 9, 10], 6)
+    s.add(b)
+    s.run()
+    assert b.generated == _expected(system + [7, 8, 9, 10], 6)    # FakeEngine checks that positions and history agree
+    assert s.n_prefix_hits == 1 and s.prefix_tokens_reused == 40
+    fed_b = sum(n for step in eng.steps for _, n in step) - fed_before
+    assert fed_b == 4 + 5                                         # only what lies beyond the shared prefix
+    # the same prompt again: everything is shared, one token is still computed (its logits are needed)
+    c = _task("c", system + [7, 8, 9, 10], 3)
+    s.add(c)
+    s.run()
+    assert c.generated == _expected(system + [7, 8, 9, 10], 3) and s.prefix_tokens_reused == 40 + 43
+    # nothing in common: a fresh cache
+    d = _task("d", [5, 4, 3], 2)
+    s.add(d)
+    s.run()
+    assert d.generated == _expected([5, 4, 3], 2) and s.n_prefix_hits == 2
+    eng.cache.check_invariants()
+    s.release_idle()
+    assert eng.cache.free_pages() == 32 and eng.cache.slots.n_free == 4 and not eng.cache.requests
+
+
+def test_kept_caches_are_given_up_before_a_running_request_is_preempted():
+    eng = FakeEngine(num_pages=8, page_size=16, max_requests=3)
+    s = Scheduler(eng, max_batch_tokens=64, chunk_size=32, prefix_cache=True)
+    first = _task("first", list(range(40)), 8)
+    s.add(first)
+    s.run()
+    assert len(s.idle) == 1 and eng.cache.free_pages() == 8 - 3
+    prompts = {"x": list(range(100, 130)), "y": list(range(200, 230))}
+    for k, p in prompts.items():
+        s.add(_task(k, p, 30))                                    # 2 x 60 tokens = 8 pages: the kept cache has to go
+    done = s.run()
+    assert s.n_preempted == 0
+    for t in done:
+        assert t.generated == _expected(prompts[t.id], 30)
+    eng.cache.check_invariants()
+    # kept caches also hold state slots: with all slots kept, a new request still gets in
+    s.release_idle()
+    for i in range(3):
+        s.add(_task("k%d" % i, [i, i + 1], 2))
+    s.run()
+    assert len(s.idle) == 3 and eng.cache.slots.n_free == 0
+    late = _task("late", [9, 9, 9], 2)
+    s.add(late)
+    s.run()
+    assert late.generated == _expected([9, 9, 9], 2)
+
+
+def test_prefix_cache_stays_off_where_keys_are_given_back():
+    from infinicore_infer_amd.cache import CacheManager, GroupSpec
+    eng = FakeEngine(num_pages=8)
+    eng.cache = CacheManager([GroupSpec("window", 1, 16, 32, (0,))], 8, 16, 4, None)
+    assert not Scheduler(eng, prefix_cache=True).prefix_cache
+    assert Scheduler(FakeEngine(num_pages=8), prefix_cache=True).prefix_cache
