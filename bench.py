@@ -3,11 +3,15 @@
 
   python bench.py --gpus 1 --steps K --warmup W
 
-A step is one decode step of the whole batch: the step function over one new
-token per request, greedy sampling on the device, and the sampled tokens fed
-back (the reference times the same loop, scripts/jiuge.py:562-583, prefill
-excluded).  Weights are random (seeded), prompts are seeded uniform-random token
-ids.  One JSON line is printed.
+A step is one decode step of the whole batch: the scheduler's step (plan, the step
+function over one new token per request, greedy sampling on the device, the sampled
+tokens fed back and the finish rules checked); the reference times the same loop,
+scripts/jiuge.py:562-583, prefill excluded.  Weights are random (seeded), prompts are
+seeded uniform-random token ids.  One JSON line is printed.
+
+  --workload mixed   the 1B shape's workload: 64 requests, prompts of 128..2,048 tokens, portions of 512
+  --workload long    the 8B shape's workload: 4 prompts of 16,384 tokens, then decoding
+  --direct           decode by calling the step function directly, without the scheduler
 """
 import argparse
 import json
@@ -78,8 +82,9 @@ def model_numbers(conf):
 
 
 def time_prefill(engine, tokens, reps=6):
+    """Mean time of a whole-prompt step with its sampled token (one untimed pass first)."""
     from infinicore_infer_amd.engine import StepEntry
-    best = None
+    total = 0.0
     for i in range(reps + 1):
         _sync()
         t0 = time.perf_counter()
@@ -89,8 +94,37 @@ def time_prefill(engine, tokens, reps=6):
         dt = time.perf_counter() - t0
         engine.free("pf")
         if i > 0:
-            best = dt if best is None else min(best, dt)
-    return best
+            total += dt
+    return total / reps
+
+
+def time_decode_scheduled(engine, batch, steps, warmup, vocab, seed=0):
+    """``batch`` requests of PROMPT tokens go through the scheduler; once all of them decode, ``warmup``
+    untimed and ``steps`` timed scheduler steps (each: one token for every request)."""
+    from infinicore_infer_amd.engine.scheduler import Scheduler
+    from infinicore_infer_amd.engine.tasks import InferTask
+    g = torch.Generator().manual_seed(seed)
+    sch = Scheduler(engine, max_batch_tokens=max(PROMPT, batch), chunk_size=PROMPT)
+    for i in range(batch):
+        toks = torch.randint(0, vocab, (PROMPT,), generator=g).tolist()
+        sch.add(InferTask("d%d" % i, toks, 1 << 30, temperature=0.0, topk=1, end_tokens=[],
+                          max_new_tokens=warmup + steps + batch + 8))     # the first ones decode while the others' prompts run
+    while sch.waiting or any(not r.decoding for r in sch.running):
+        sch.step()
+    for _ in range(warmup):
+        assert len(sch.step()) == batch
+    _sync()
+    ctx0 = engine.length("d0")
+    t0 = time.perf_counter()
+    for _ in range(steps):
+        sch.step()
+    _sync()
+    dt = time.perf_counter() - t0
+    ctx1 = engine.length("d0")
+    assert len(sch.running) == batch and sch.n_preempted == 0
+    for i in range(batch):
+        sch.abort("d%d" % i)
+    return dt / steps, (ctx0 + ctx1) / 2.0
 
 
 def time_decode(engine, batch, steps, warmup, vocab, seed=0):
@@ -179,6 +213,21 @@ def run_mixed(args):
         "decode_steps": {"count": len(dec), "mean_ms": round(1e3 * sum(s[0] for s in dec) / max(1, len(dec)), 3)},
         "preempted": preempted,
     }
+    weight_bytes, kv_per_tok, prefill_flops = model_numbers(conf)
+    if mixed:      # a mixed step's matrix-product flops (its prompt portions dominate) against the bf16 peak
+        d, L, di = conf.hidden_size, conf.num_hidden_layers, conf.intermediate_size
+        per_tok = 2.0 * L * ((conf.num_attention_heads + 2 * conf.num_key_value_heads) * conf.head_dim * d
+                             + conf.num_attention_heads * conf.head_dim * d + 3 * d * di)
+        t_mixed = sum(s[0] for s in mixed) / len(mixed)
+        n_mixed = sum(s[1] for s in mixed) / len(mixed)
+        out["prefill"] = {"value": round(n_mixed / t_mixed, 1), "tokens": round(n_mixed, 1), "ms": round(t_mixed * 1e3, 3),
+                          "frac": round(per_tok * n_mixed / t_mixed / (PEAK_TFLOPS["bf16"] * 1e12), 4)}
+    if dec:        # a decode-only step reads every weight once and the live requests' cache
+        t_dec = sum(s[0] for s in dec) / len(dec)
+        ctx_mean = sum(lens) / len(lens) + gen / 2.0
+        achieved = (weight_bytes + n_req * ctx_mean * kv_per_tok) / t_dec / 1e9
+        out["roofline"] = {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
+                           "frac": round(achieved / HBM_PEAK_GBS, 4)}
     print(json.dumps(out))
     return 0
 
@@ -191,9 +240,11 @@ def main():
     ap.add_argument("--warmup", type=int, default=16)
     ap.add_argument("--layers", type=int, default=0, help="fewer layers than the shape has (0: all)")
     ap.add_argument("--shape", default=None, choices=sorted(SHAPES), help="2b is the benchmark's configuration (default; 1b for --workload mixed)")
-    ap.add_argument("--workload", default="decode", choices=["decode", "mixed"],
+    ap.add_argument("--workload", default="decode", choices=["decode", "mixed", "long"],
                     help="decode: the benchmark (prefill of one prompt, decode steps at fixed batches); "
-                         "mixed: 64 requests of 128..2048 prompt tokens through the scheduler, --steps tokens generated each")
+                         "mixed: 64 requests of 128..2048 prompt tokens through the scheduler, --steps tokens generated each; "
+                         "long: the 8B shape with 4 prompts of 16,384 tokens (the same as --shape 8b --prompt 16384 --batch 4 --no-points)")
+    ap.add_argument("--direct", action="store_true", help="decode through the step function directly, not through the scheduler")
     ap.add_argument("--requests", type=int, default=64, help="--workload mixed: number of requests")
     ap.add_argument("--token-budget", type=int, default=1024, help="--workload mixed: tokens per step")
     ap.add_argument("--prompt", type=int, default=PROMPT)
@@ -208,6 +259,13 @@ def main():
         return 2
 
     sys.path.insert(0, os.path.dirname(os.path.abspath(__file__)))
+    if args.workload == "long":
+        args.shape = args.shape or "8b"
+        if args.prompt == ap.get_default("prompt"):
+            args.prompt = 16384
+        if args.batch == ap.get_default("batch"):
+            args.batch = 4
+        args.no_points = True
     if args.shape is None:
         args.shape = "1b" if args.workload == "mixed" else "2b"
     MODEL, PROMPT = SHAPES[args.shape], args.prompt
@@ -215,7 +273,7 @@ def main():
         if args.steps == ap.get_default("steps"):
             args.steps = 64
         return run_mixed(args)
-    per_req = PROMPT + args.warmup + args.steps + 64
+    per_req = PROMPT + args.warmup + args.steps + 64 + max(BATCH, args.batch, 64)
     per_req = (per_req + 63) // 64 * 64
     BATCH = args.batch
     batches = [BATCH] if args.no_points else sorted({BATCH, 1, 64}, key=lambda b: (b != BATCH, b))
@@ -234,8 +292,9 @@ def main():
     pf_flops = prefill_flops(PROMPT)
 
     results = {}
+    decode = time_decode if args.direct else time_decode_scheduled
     for b in batches:
-        results[b] = time_decode(engine, b, args.steps, args.warmup, vocab, seed=b)
+        results[b] = decode(engine, b, args.steps, args.warmup, vocab, seed=b)
     ms, ctx = results[BATCH][0] * 1e3, results[BATCH][1]
     value = BATCH / results[BATCH][0]
     bytes_step = weight_bytes + BATCH * ctx * kv_per_tok
@@ -253,7 +312,7 @@ def main():
             "global_batch": BATCH, "seq_len": PROMPT, "context_mean": round(ctx, 1), "generated": args.steps,
             "page_size": args.page_size, "tied_embeddings": bool(MODEL.get("tie_word_embeddings", True)), "parallelism": "single-gpu",
             "sampling": "greedy on device", "library_gemm": "default" if args.no_tune else "algorithms timed per shape",
-            "decode_launch": "eager" if args.eager else "hip graph",
+            "decode_launch": "eager" if args.eager else "hip graph", "decode_loop": "direct" if args.direct else "scheduler",
         },
         "prefill": {"value": round(PROMPT / t_pf, 1), "tokens": PROMPT, "ms": round(t_pf * 1e3, 3),
                     "frac": round(pf_flops / t_pf / (PEAK_TFLOPS["bf16"] * 1e12), 4)},

@@ -163,8 +163,25 @@ class Scheduler:
         budget = self.max_batch_tokens
         plan: List[Tuple[_Running, int]] = []
 
-        # 1. decodes, oldest first; preempt the youngest when pages run out
-        for r in sorted([r for r in self.running if r.decoding], key=lambda r: r.order):
+        # 1. decodes, oldest first; preempt the youngest when pages run out.  The usual case first, in one pass:
+        # every decoding request gets its token and the pages for them are there (``running`` is in admission
+        # order: requests are appended when admitted and a preempted one is admitted anew).
+        decoding = [r for r in self.running if r.decoding]
+        if decoding and len(decoding) <= budget:
+            ps, reqs = self.cache.page_size, self.cache.requests
+            need = [0] * ngroups
+            for r in decoding:
+                e = reqs[r.task.id]
+                pages = e.length // ps + 1
+                for g, table in enumerate(e.tables):
+                    if len(table) < pages:
+                        need[g] += pages - len(table)
+            if self._fits(need, reserved):
+                reserved = need
+                plan = [(r, 1) for r in decoding]
+                budget -= len(decoding)
+                decoding = []
+        for r in sorted(decoding, key=lambda r: r.order):
             if r not in self.running or budget < 1:
                 continue
             while True:
