@@ -14,6 +14,9 @@
 // k-steps when at most 16 / AG rows are in use (the spare lanes carry the other
 // steps' data and a row rotation hands it over).
 //
+// With 32,768 weight rows or more and up to 16 rows of A (the output head) a second kernel runs, in which
+// waves own whole weight tiles (gemm_wide_kernel below).
+//
 // 16x16x32 layout (lane l): A[i = l%16][k = 8(l/16)..+7], B[k = 8(l/16)..+7][j = l%16],
 // D[i = 4(l/16) + e][j = l%16], e = 0..3.
 #include "common.h"
@@ -410,6 +413,176 @@ static int compute_units() {
     return cus;
 }
 
+// Very many weight rows and at most 16 token rows (the output head over the vocabulary): there are enough 16-row
+// weight tiles for every wave to own whole tiles, so nothing is summed across waves.  The token rows are staged in
+// LDS once per block (zero-filled beyond K; rows padded by 16 bytes so that 8 rows hit different banks); a wave
+// walks K in groups of kWideDepth k-steps, with the next group's loads (of the same or of its next tile) issued
+// before the current group is used, so its weight stream never pauses between tiles.  A block owns a run of whole
+// tiles and its waves equal shares of the run's (tile, group) pairs, so that every wave reads the same number of
+// bytes; where a share ends inside a tile, the two waves that hold the tile's halves add them through LDS.
+constexpr int kWideDepth = 8;
+constexpr int kWideLdsLimit = 160 * 1024;             // LDS of a compute unit
+
+// WV waves a block: 8 when two blocks' token rows fit a compute unit's LDS, else 16 in one block
+template <typename TC, int WV>
+__global__ void __launch_bounds__(WV * 64)
+gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
+                 int lda, int ldw, int ldc, float alpha, NormFuse nf, int a_stride) {
+    extern __shared__ __align__(16) unsigned char wide_smem[];
+    uint16_t* As = reinterpret_cast<uint16_t*>(wide_smem);                       // [M][a_stride]
+    float* part = reinterpret_cast<float*>(wide_smem + (size_t)M * a_stride * 2);    // [4 WV][16]
+    float* rowf_s = part + 4 * WV * 16;                                          // [16]
+    v4f* heads = reinterpret_cast<v4f*>(rowf_s + 16);                            // [WV][64]
+    const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, kq = lane >> 4;
+    const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
+    constexpr int D = kWideDepth;
+    const int steps = (K + 31) >> 5, groups = (steps + D - 1) / D, tiles = (N + 15) >> 4;
+    // the block's tiles, and this wave's run of (tile, group) pairs among them
+    const int t0 = (int)((long long)blockIdx.x * tiles / gridDim.x), t1 = (int)((long long)(blockIdx.x + 1) * tiles / gridDim.x);
+    const int bg = (t1 - t0) * groups;
+    const int run0 = (int)((long long)wave * bg / WV), total = (int)((long long)(wave + 1) * bg / WV) - run0;
+    const int klast = K - 8;                                 // the last whole 16 bytes of a weight row
+    // group L of this wave's run (clamped to its last one, so that loads are never conditional): weights only;
+    // columns beyond K repeat the row's last 16 bytes and meet zeros of the staged token rows
+    auto issue = [&](uint4 (&w)[D], int L) {
+        L = run0 + (L < total ? L : total - 1);
+        const int ti = L / groups, g = L - ti * groups;
+        const int n = (t0 + ti) * 16 + r;
+        const uint16_t* p = W + (size_t)(n < N ? n : N - 1) * ldw;
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            const int k = 32 * (g * D + u) + 8 * kq;
+            w[u] = *reinterpret_cast<const uint4*>(p + (k < klast ? k : klast));
+        }
+    };
+    uint4 w0[D], w1[D];
+    if (total > 0) issue(w0, 0);                             // the weights do not wait for the token rows
+    const int chunks = a_stride >> 3;                        // 16-byte pieces of a staged row
+    for (int m = wave; m < M; m += WV) {                     // a wave stages whole rows, four loads at a time
+        const uint16_t* src = A + (size_t)m * lda;
+        uint16_t* dst = As + (size_t)m * a_stride;
+        for (int c0 = lane; c0 < chunks; c0 += 256) {
+            uint4 v[4];
+#pragma unroll
+            for (int j = 0; j < 4; ++j) {
+                const int c = c0 + 64 * j;
+                v[j] = make_uint4(0u, 0u, 0u, 0u);
+                if (8 * c + 8 <= K) v[j] = *reinterpret_cast<const uint4*>(src + 8 * c);
+            }
+#pragma unroll
+            for (int j = 0; j < 4; ++j)
+                if (c0 + 64 * j < chunks) *reinterpret_cast<uint4*>(dst + 8 * (c0 + 64 * j)) = v[j];
+        }
+    }
+    if (nf.ss_in) {
+        float t = 0.f;
+        for (int b = tid >> 4; b < nf.n_parts_in; b += 4 * WV) t += nf.ss_in[b * 16 + (tid & 15)];
+        part[(tid >> 4) * 16 + (tid & 15)] = t;
+    }
+    __syncthreads();
+    if (tid < 16) {
+        float f = 1.0f;
+        if (nf.ss_in) {
+            float t = 0.f;
+            for (int j = 0; j < 4 * WV; ++j) t += part[j * 16 + tid];
+            f = rsqrtf(t * nf.inv_width + nf.eps);
+        }
+        rowf_s[tid] = f;
+    }
+    __syncthreads();
+    const float scale = alpha * rowf_s[r];                   // column j = r of D is token row r
+    const uint16_t* arow = As + (size_t)(r < M ? r : M - 1) * a_stride + 8 * kq;
+
+    // D[i = 4 kq + e][j = r]: weight row 16 tile + 4 kq + e, token row r
+    auto store = [&](int tile, const v4f& v) {
+        if (r < M) {
+#pragma unroll
+            for (int e = 0; e < 4; ++e) {
+                const int n = tile * 16 + 4 * kq + e;
+                if (n < N) C[(size_t)r * ldc + n] = from_f32<TC>(scale * v[e]);
+            }
+        }
+    };
+    v4f acc = v4f{0.f, 0.f, 0.f, 0.f}, tail_acc = acc;
+    int ct = t0 + run0 / groups, cg = run0 - (run0 / groups) * groups;       // tile and group the next use belongs to
+    // A run that begins inside a tile holds that tile's tail; its head is the end of the previous wave's run.
+    const bool has_tail = total > 0 && cg != 0;
+    const int tail_tile = ct;
+    bool in_tail = has_tail;
+    auto use = [&](const uint4 (&w)[D]) {
+        typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+#pragma unroll
+        for (int u = 0; u < D; ++u) {
+            const uint4 a = *reinterpret_cast<const uint4*>(arow + 32 * (cg * D + u));
+            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w[u]), __builtin_bit_cast(v8b, a), acc, 0, 0, 0);
+        }
+        if (++cg == groups) {
+            if (in_tail) { tail_acc = acc; in_tail = false; }
+            else store(ct, acc);
+            acc = v4f{0.f, 0.f, 0.f, 0.f};
+            cg = 0;
+            ++ct;
+        }
+    };
+    for (int L = 0; L < total; L += 2) {
+        issue(w1, L + 1);
+        use(w0);
+        issue(w0, L + 2);
+        if (L + 1 < total) use(w1);
+    }
+    // The launcher gives every wave at least `groups` pairs, so a tile is shared by two waves at most: the head
+    // goes through LDS to the wave that holds the tail, which adds the two in this order and stores.
+    if (total > 0 && cg != 0) heads[wave * 64 + lane] = acc;
+    __syncthreads();
+    if (has_tail) {
+        const v4f h = heads[(wave - 1) * 64 + lane];
+        store(tail_tile, h + tail_acc);
+    }
+}
+
+static bool g_wide_enabled = true;
+// For measurements: 0 sends wide products through the tiled kernel again.  Returns the previous setting.
+IC_EXPORT int ic_gemm_nt_wide_enable(int on) { const int was = g_wide_enabled; g_wide_enabled = on != 0; return was; }
+
+// false when the wide kernel does not take the shape.
+template <typename TC>
+static bool launch_gemm_wide(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
+                             float alpha, const NormFuse& nf, hipStream_t stream) {
+    const int steps = (K + 31) / 32, groups = (steps + kWideDepth - 1) / kWideDepth;
+    const int a_stride = groups * kWideDepth * 32 + 8;
+    const size_t rows_bytes = (size_t)M * a_stride * 2;
+    auto lds_of = [&](int wv) { return rows_bytes + (4 * wv * 16 + 16) * sizeof(float) + (size_t)wv * 64 * 16; };
+    // two blocks of 8 waves a compute unit; with many or long token rows one block of 16 waves, or of 8 when only that fits
+    const bool two = 2 * lds_of(8) <= (size_t)kWideLdsLimit;
+    const int wv = (two || lds_of(16) > (size_t)kWideLdsLimit) ? 8 : 16;
+    const size_t lds = lds_of(wv);
+    if (M > 16 || K < 8 || K % 8 || lds > (size_t)kWideLdsLimit) return false;
+    static bool raised[2][2][64] = {};                       // per kernel and device: it may use more than 64 KB of LDS
+    int dev = 0;
+    if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
+    bool& done = raised[sizeof(TC) == 2 ? 1 : 0][wv == 8 ? 1 : 0][dev];
+    const void* fn = wv == 8 ? (const void*)gemm_wide_kernel<TC, 8> : (const void*)gemm_wide_kernel<TC, 16>;
+    if (!done) {
+        if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kWideLdsLimit) != hipSuccess) {
+            (void)hipGetLastError();
+            return false;
+        }
+        done = true;
+    }
+    // as many blocks as are resident at once, each with a whole number of tiles and at least one tile per wave
+    const int tiles = (N + 15) / 16, cus = compute_units();
+    int blocks = cus * (two ? 2 : 1);
+    if (blocks > tiles / wv) blocks = tiles / wv;
+    if (blocks < 1) return false;
+    if (wv == 8)
+        hipLaunchKernelGGL((gemm_wide_kernel<TC, 8>), dim3(blocks), dim3(512), lds, stream, (const uint16_t*)A,
+                           (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, nf, a_stride);
+    else
+        hipLaunchKernelGGL((gemm_wide_kernel<TC, 16>), dim3(blocks), dim3(1024), lds, stream, (const uint16_t*)A,
+                           (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, nf, a_stride);
+    return true;
+}
+
 // NT weight tiles of 16 rows share one load of the A fragments; WPB waves split K.  Both are
 // chosen so that (column blocks x waves) fills the chip's SIMDs about twice over.
 template <typename TC>
@@ -418,6 +591,8 @@ static void dispatch_gemm(const void* A, const void* W, void* C, int M, int N, i
     const int tiles = (N + 15) / 16;
 #define IC_GO(NT, MT, WPB, UN) launch_gemm<TC, NT, MT, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream)
     // tilings from a sweep over the projection shapes of 1B..8B models on MI355X
+    if (M <= 16 && tiles >= 2048 && aligned && g_wide_enabled &&
+        launch_gemm_wide<TC>(A, W, C, M, N, K, lda, ldw, ldc, alpha, nf, stream)) return;
     if (M <= 16) {
         if (tiles < 400) IC_GO(1, 1, 16, 4);
         else if (tiles < 600) IC_GO(2, 1, 16, 4);

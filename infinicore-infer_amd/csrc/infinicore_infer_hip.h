@@ -74,6 +74,9 @@ typedef struct {
 int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype);
 int ic_gemm_nt_residual_parts(int N);
 int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode, const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream);
+// Products of up to 16 rows with 32,768 weight rows or more (the output head) run in a kernel whose waves own whole
+// weight tiles; 0 sends them through the tiled kernel instead (for measurements).  Returns the previous setting.
+int ic_gemm_nt_wide_enable(int on);
 // The same with the tiling chosen by the caller (tuning and tests); nt == 0 selects the SwiGLU variant.
 int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int nt, int wpb, int unroll, hipStream_t stream);
 // QKV projection of M <= 16 rows with rotary and cache write in the epilogue; row_factor nullable.

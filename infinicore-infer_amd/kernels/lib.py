@@ -108,6 +108,7 @@ _SIGNATURES = {
     "ic_argmax_static": [_P, _LL, _I, _I, _P, _P],
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],
     "ic_gemm_nt_residual_parts": [_I],
+    "ic_gemm_nt_wide_enable": [_I],
     "ic_gemm_nt_supported": [_I, _I, _I],
     "ic_gemm_qkv_rope_supported": [_I, _I],
     "ic_gemm_qkv_rope": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _RF, _P],

@@ -335,7 +335,10 @@ def test_attention_far_key_and_window_edge(impl, dtype):
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("cdtype", DT)
 @pytest.mark.parametrize("M,N,K", [(1, 331, 200), (8, 2304, 2304), (16, 509, 96), (17, 1000, 344), (64, 777, 5760),
-                                   (3, 122753, 64), (130, 300, 100)])
+                                   (3, 122753, 64), (130, 300, 100),
+                                   # 32,768 weight rows and more with up to 16 rows: waves own whole weight tiles;
+                                   # 8 waves a block, 16 where the token rows take most of the LDS, few groups of K
+                                   (7, 50007, 2304), (16, 35001, 1032), (13, 40000, 4104), (1, 33000, 8)])
 def test_gemm_nt(cdtype, M, N, K):
     g = torch.Generator().manual_seed(16)
     a = torch.randn(M, K, generator=g).to(torch.bfloat16)
@@ -530,7 +533,8 @@ def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page, tile_rows):
 
 
 @pytest.mark.parametrize("M,N,K,N2", [(1, 200, 344, 331), (8, 2304, 2304, 6912), (16, 96, 509, 64), (5, 4096, 130, 50),
-                                      (3, 1536, 3840, 1000), (7, 304, 8264, 130), (16, 512, 16384, 96)])
+                                      (3, 1536, 3840, 1000), (7, 304, 8264, 130), (16, 512, 16384, 96),
+                                      (5, 200, 344, 33331), (16, 1000, 72, 40002)])
 def test_norm_split_over_two_products(M, N, K, N2):
     """Residual add + RMS norm between two products, split over them: the first product's
     epilogue adds to the stream and stores x * w with sums of squares; the second applies the
