@@ -129,31 +129,54 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     // lookup per tile and every load is that tile's first row plus an offset the thread keeps.
     constexpr int KPI = kPfThreads / (DH / 8);                // keys one pass of K loads covers (<= 64)
     static_assert(KPI <= kPfKeys && kPfKeys % KPI == 0, "a pass of loads stays inside a tile");
+    // what a thread loads in a step never changes: key `tkey` of the step's keys, at element `toff` of its 64-key tile
+    int tkey[NL];
+    uint32_t toff[NL];
+#pragma unroll
+    for (int i = 0; i < NL; ++i) {
+        const int idx = tid + i * kPfThreads;
+        const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
+        tkey[i] = key;
+        toff[i] = (uint32_t)(((key % kPfKeys) * DH + oct * 8) * sizeof(uint16_t));
+    }
     auto fetch = [&](int kt) {
-        size_t tile_row[GROUPS];                              // PAGE64: element offset of each tile's first row
         if (PAGE64) {
+            // one page lookup per tile, the same for every lane: the tile's first row is a scalar address and a load
+            // adds the thread's constant offset to it
+            const char* krow[GROUPS];
+            const char* vrow[GROUPS];
 #pragma unroll
             for (int t = 0; t < GROUPS; ++t) {
                 const int k0 = kt + kPfKeys * t;
                 const int k0c = (k0 <= last_key) ? k0 : last_key;     // a tile beyond the end is not loaded at all
-                tile_row[t] = (size_t)page_of(k0c) * page_stride + (size_t)(k0 & page_mask) * DH;
+                const int pg = __builtin_amdgcn_readfirstlane(page_of(k0c));
+                const size_t row = (size_t)pg * page_stride + (size_t)(k0 & page_mask) * DH;
+                krow[t] = reinterpret_cast<const char*>(kbase + row);
+                vrow[t] = reinterpret_cast<const char*>(vbase + row);
             }
+#pragma unroll
+            for (int i = 0; i < NL; ++i) {
+                const int ka = kt + tkey[i];
+                kreg[i] = make_uint4(0, 0, 0, 0);
+                vreg[i] = make_uint4(0, 0, 0, 0);
+                if (ka <= last_key && ka >= first_key) {
+                    kreg[i] = *reinterpret_cast<const uint4*>(krow[(i * KPI) / kPfKeys] + toff[i]);
+                    vreg[i] = *reinterpret_cast<const uint4*>(vrow[(i * KPI) / kPfKeys] + toff[i]);
+                }
+            }
+            return;
         }
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
             const int idx = tid + i * kPfThreads;
-            {
-                const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
-                const int ka = kt + key;
-                kreg[i] = make_uint4(0, 0, 0, 0);
-                vreg[i] = make_uint4(0, 0, 0, 0);
-                if (ka <= last_key && ka >= first_key) {
-                    size_t off;
-                    if (PAGE64) off = tile_row[(i * KPI) / kPfKeys] + (size_t)(key % kPfKeys) * DH + oct * 8;
-                    else off = (size_t)page_of(ka) * page_stride + (size_t)(ka & page_mask) * DH + oct * 8;
-                    kreg[i] = *reinterpret_cast<const uint4*>(kbase + off);
-                    vreg[i] = *reinterpret_cast<const uint4*>(vbase + off);
-                }
+            const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
+            const int ka = kt + key;
+            kreg[i] = make_uint4(0, 0, 0, 0);
+            vreg[i] = make_uint4(0, 0, 0, 0);
+            if (ka <= last_key && ka >= first_key) {
+                const size_t off = (size_t)page_of(ka) * page_stride + (size_t)(ka & page_mask) * DH + oct * 8;
+                kreg[i] = *reinterpret_cast<const uint4*>(kbase + off);
+                vreg[i] = *reinterpret_cast<const uint4*>(vbase + off);
             }
         }
     };
@@ -197,15 +220,20 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         // ---- mask (only tiles that touch the diagonal or the window's edge) -----------
         const bool need_mask = (kt + kPfKeys - 1 > wave_first) || (window > 0);
         if (need_mask) {
+            // key kt + 4 half + e of this lane's accumulator (e a constant per accumulator) is seen when e <= lim
+            const int lim = qpos - kt - 4 * half;
 #pragma unroll
             for (int tt = 0; tt < 2; ++tt)
 #pragma unroll
-                for (int r = 0; r < 16; ++r) {
-                    const int ka = kt + 32 * tt + 8 * (r >> 2) + 4 * half + (r & 3);
-                    bool ok = ka <= qpos;
-                    if (window > 0) ok = ok && (ka > qpos - window);
-                    if (!ok) sacc[tt][r] = -INFINITY;
-                }
+                for (int r = 0; r < 16; ++r)
+                    if (32 * tt + 8 * (r >> 2) + (r & 3) > lim) sacc[tt][r] = -INFINITY;
+            if (window > 0) {
+#pragma unroll
+                for (int tt = 0; tt < 2; ++tt)
+#pragma unroll
+                    for (int r = 0; r < 16; ++r)
+                        if (32 * tt + 8 * (r >> 2) + (r & 3) <= lim - window) sacc[tt][r] = -INFINITY;
+            }
         }
         // ---- running softmax, base 2: p = 2^(s c - m c) ---------------------------------
         float mloc = sacc[0][0];
