@@ -239,7 +239,7 @@ def _parse(argv):
     ap.add_argument("--prompt", default=None, help="a text prompt (needs a tokenizer in the model folder)")
     ap.add_argument("--prompt-ids", action="append", default=None,
                     help="a prompt as comma-separated token ids; may be given several times")
-    ap.add_argument("--prompt-len", type=int, default=None, help="random token ids of this length as the prompt")
+    ap.add_argument("--prompt-len", type=int, default=None, help="random token ids of this length as the prompt (the first is bos_token_id if the configuration has one)")
     ap.add_argument("--num-prompts", type=int, default=1, help="with --prompt-len: how many such prompts")
     ap.add_argument("--max-new-tokens", "--max-steps", dest="max_new_tokens", type=int, default=500)
     ap.add_argument("--temperature", type=float, default=1.0)
@@ -292,8 +292,11 @@ def test(argv=None):
     if args.prompt_ids:
         prompts = [[int(t) for t in p.split(",") if t.strip()] for p in args.prompt_ids]
     elif args.prompt_len:
+        # as a tokenizer would: the configuration's bos token first, when it names one
         rng = random.Random(args.seed)
-        prompts = [[rng.randrange(model.config.vocab_size) for _ in range(args.prompt_len)]
+        bos = getattr(model.config, "bos_token_id", None)
+        head = [int(bos)] if isinstance(bos, int) and 0 <= bos < model.config.vocab_size else []
+        prompts = [(head + [rng.randrange(model.config.vocab_size) for _ in range(args.prompt_len)])[:args.prompt_len]
                    for _ in range(args.num_prompts)]
     else:
         prompts = [args.prompt if args.prompt is not None else "山东最高的山是？"]

@@ -180,6 +180,33 @@ def test_embedding_and_head_parts():
     assert logits.dtype == torch.float32 and _rel(logits, P.plain_linear(hn, table)) < 2e-3
 
 
+def test_weights_drawn_on_the_device_are_the_folder_written_on_the_cpu(tmp_path_factory):
+    """Random-weights mode both ways: a folder written on the CPU and loaded, and weights drawn straight into a
+    model on the GPU.  One seed, one model: every tensor is equal bit for bit, and so are the logits."""
+    from infinicore_infer_amd.config import config_from_dict
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    from infinicore_infer_amd.parts import Runtime, build_model
+    from infinicore_infer_amd.weights import init_random_weights, standard_normal, write_random_model
+    z = standard_normal(5, "model.embed_tokens.weight", 300001, device=DEV)
+    assert torch.equal(z.cpu(), standard_normal(5, "model.embed_tokens.weight", 300001))
+    for name, cfg, init in (("A", H.TINY_A, H.TINY_A_INIT), ("B", H.TINY_B, H.TINY_B_INIT)):
+        folder = write_random_model(str(tmp_path_factory.mktemp("drawn_" + name)), cfg, seed=21, **init)
+        loaded = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=64)
+        model = build_model(config_from_dict(cfg).model_spec(), Runtime(torch.bfloat16, DEV))
+        init_random_weights(model, seed=21, tie=cfg.get("tie_word_embeddings", True), **init)
+        drawn = Engine(model, max_tokens=64)
+        la, lb = loaded.model.layers[-1], drawn.model.layers[-1]
+        for x, y in ((loaded.model.embedding.table, drawn.model.embedding.table), (loaded.model.head.weight, drawn.model.head.weight),
+                     (la.mixer.w_qkv, lb.mixer.w_qkv), (la.mixer.w_o, lb.mixer.w_o), (la.feed_forward.w_gate_up, lb.feed_forward.w_gate_up),
+                     (la.feed_forward.w_down, lb.feed_forward.w_down), (la.feed_forward_norm.weight, lb.feed_forward_norm.weight),
+                     (loaded.model.final_norm.weight, drawn.model.final_norm.weight)):
+            assert x.dtype == y.dtype and torch.equal(x, y)
+        toks = [3, 1, 4, 1, 5, 9, 2, 6]
+        a = loaded.step([StepEntry("r", toks, list(range(len(toks))))])
+        b = drawn.step([StepEntry("r", toks, list(range(len(toks))))])
+        assert torch.equal(a, b)
+
+
 # ---------------------------------------------------------------------------
 # generation through the entry point and the scheduler
 # ---------------------------------------------------------------------------

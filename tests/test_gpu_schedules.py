@@ -259,11 +259,14 @@ def test_preemption_under_temperature_sampling_gives_the_same_tokens(tmp_path_fa
     if dtype == torch.float32:
         assert tight == plenty
     else:
-        # bfloat16: a recomputed prompt runs as portions where it ran token by token before, which moves
-        # logits by rounding; a draw that falls on a boundary may then choose a neighbour, and the
-        # continuation differs from there on.  The requests never preempted must be identical.
-        same = sum(a == b for a, b in zip(tight, plenty))
-        assert same >= 1 and tight[0] == plenty[0]
+        # bfloat16: with other requests beside it a row runs through other kernels (more rows, other key splits),
+        # and a recomputed prompt runs as portions where it ran token by token before: logits move by rounding,
+        # a draw that falls on a boundary of the cumulative distribution may then choose the neighbour, and the
+        # continuation differs from there on.  The draws are the same numbers, so the two runs agree until such a
+        # boundary is hit: long common beginnings, not equality.
+        common = [next((i for i, (x, y) in enumerate(zip(a, b)) if x != y), len(a)) for a, b in zip(tight, plenty)]
+        print("tokens in common before the first difference:", common)
+        assert sum(common) >= 40 and max(common) >= 20
 
 
 # ---- the command line ---------------------------------------------------------------------------------------------------

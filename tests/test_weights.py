@@ -41,6 +41,45 @@ def test_random_folder_loads_and_is_reproducible(tmp_path):
     assert float(load_file(os.path.join(b, "model.safetensors"))["model.norm.weight"].float().std()) > 0.05
 
 
+def _numpy_standard_normal(seed, name, n):
+    """The draw written out a second time, with numpy's unsigned integers: two splitmix64-finalised words per element,
+    eight 16-bit uniforms, their centred sum times sqrt(12 / 8)."""
+    import hashlib
+    import numpy as np
+    key = int.from_bytes(hashlib.sha256(("%d:%s" % (seed, name)).encode()).digest()[:8], "little")
+    i = np.arange(n, dtype=np.uint64)
+    total = np.zeros(n, dtype=np.int64)
+    with np.errstate(over="ignore"):
+        for word in (0, 1):
+            x = i * np.uint64(0x9E3779B97F4A7C15) + np.uint64((key + word * 0x94D049BB133111EB) % (1 << 64))
+            x ^= x >> np.uint64(30)
+            x *= np.uint64(0xBF58476D1CE4E5B9)
+            x ^= x >> np.uint64(27)
+            x *= np.uint64(0x94D049BB133111EB)
+            x ^= x >> np.uint64(31)
+            for field in range(4):
+                total += ((x >> np.uint64(16 * field)) & np.uint64(0xFFFF)).astype(np.int64)
+    return ((total - (4 * 65536 - 4)).astype(np.float64) * ((1.5 ** 0.5) / 65536.0)).astype(np.float32)
+
+
+def test_a_random_value_depends_on_seed_name_and_index_only(monkeypatch):
+    from infinicore_infer_amd.weights import random_init, standard_normal
+    name = "model.layers.3.mlp.up_proj.weight"
+    z = standard_normal(7, name, 200000)
+    assert torch.equal(z, torch.from_numpy(_numpy_standard_normal(7, name, 200000)))
+    # close to a standard normal: mean, variance, fourth moment (Irwin-Hall with n = 8 has kurtosis 3 - 0.15), tails
+    assert abs(float(z.mean())) < 0.01 and abs(float(z.var()) - 1.0) < 0.01
+    assert abs(float((z ** 4).mean()) - 2.85) < 0.1 and 3.5 < float(z.abs().max()) < 4.9
+    # a prefix is a prefix, whatever the pieces it is drawn in
+    monkeypatch.setattr(random_init, "_CHUNK", 777)
+    assert torch.equal(standard_normal(7, name, 5000), z[:5000])
+    # other seed, other name: other values, uncorrelated
+    for other in (standard_normal(8, name, 200000), standard_normal(7, name + "x", 200000)):
+        assert abs(float((other * z).mean())) < 0.01
+    # neighbouring elements are uncorrelated too
+    assert abs(float((z[1:] * z[:-1]).mean())) < 0.01
+
+
 def test_dtype_rules(tmp_path):
     folder = H.make_model_dir(tmp_path, "A", seed=1)
     m32 = _model("A", torch.float32)
