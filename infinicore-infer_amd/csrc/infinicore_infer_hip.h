@@ -122,6 +122,13 @@ int ic_argmax_static(const float* logits, long long row_stride, int n_rows, int 
 // Temperature / top-k / top-p with one uniform draw per row; temperature == nullptr: argmax.
 int ic_sample(const float* logits, long long row_stride, int n_rows, int V, const float* temperature, const int* top_k, const float* top_p, const float* uniform, int* out, hipStream_t stream);
 
+// ---- what the device reaches at most (measurements for the reports, not on the model's path) ------------------------
+// Issues only MFMA instructions (bfloat16, 32x32x16) on blocks_per_unit blocks of four waves per compute unit; returns
+// the floating-point operations issued (the caller times the launch), or a negative status.
+long long ic_peak_mfma_bf16(float* sink, int iters, int blocks_per_unit, hipStream_t stream);
+// Reads `bytes` of device memory once with 16-byte loads and does nothing else.
+int ic_peak_read(const void* src, long long bytes, int blocks_per_unit, unsigned* sink, hipStream_t stream);
+
 #ifdef __cplusplus
 }
 #endif

@@ -109,6 +109,8 @@ _SIGNATURES = {
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],
     "ic_gemm_nt_residual_parts": [_I],
     "ic_gemm_nt_wide_enable": [_I],
+    "ic_peak_mfma_bf16": [_P, _I, _I, _P],
+    "ic_peak_read": [_P, _LL, _I, _P, _P],
     "ic_gemm_nt_supported": [_I, _I, _I],
     "ic_gemm_qkv_rope_supported": [_I, _I],
     "ic_gemm_qkv_rope": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _RF, _P],
@@ -134,7 +136,8 @@ _SIGNATURES = {
     "ic_decoder_step": [_P, _c.POINTER(IcHostBatch), _P, _P, _LL, _P, _LL, _P, _LL, _P, _c.POINTER(IcStepBatch), _P],
 }
 _RESTYPES = {"ic_decoder_create": _P, "ic_decoder_create_error": _c.c_char_p, "ic_decoder_destroy": None,
-             "ic_decoder_last_error": _c.c_char_p, "ic_decoder_workspace_bytes": _LL, "ic_decoder_step_ints": _LL}
+             "ic_decoder_last_error": _c.c_char_p, "ic_decoder_workspace_bytes": _LL, "ic_decoder_step_ints": _LL,
+             "ic_peak_mfma_bf16": _LL}
 
 
 def get_lib():

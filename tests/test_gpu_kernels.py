@@ -658,3 +658,11 @@ def test_gemm_in_slices_refuses_what_it_does_not_take():
         ops.gemm_splitk(a[:8], w, torch.empty(2 * 8 * 64, device=DEV), 2)
     assert not ops.gemm_splitk_pays(16, 2304, 2304) and not ops.gemm_splitk_pays(65, 2304, 2304)
     assert not ops.gemm_splitk_pays(32, 200, 344)                     # too few blocks for the chip
+
+
+def test_the_device_peak_measurements_run():
+    """The kernels that measure what the matrix cores and the memory deliver when nothing else is done: they run, and
+    their figures are of the right order (not a check of the hardware: bounds far from the expected 2,400 and 6)."""
+    from infinicore_infer_amd.kernels import peaks
+    assert 500 < peaks.mfma_bf16_tflops(iters=2000, blocks_per_unit=4) < 5100
+    assert 1.0 < peaks.read_tbs(megabytes=512, blocks_per_unit=8) < 16.5
