@@ -29,7 +29,8 @@ _M64 = (1 << 64) - 1
 _GOLDEN = 0x9E3779B97F4A7C15
 _MIX1 = 0xBF58476D1CE4E5B9
 _MIX2 = 0x94D049BB133111EB
-_CHUNK = 1 << 24                                        # elements drawn at a time (bounds the temporaries)
+_CHUNK = 1 << 24                                        # elements drawn at a time on a GPU (bounds the temporaries)
+_CHUNK_CPU = 1 << 18                                    # on the CPU: pieces that stay in its caches (20 times faster)
 
 
 def _key(seed: int, name: str) -> int:
@@ -61,8 +62,9 @@ def standard_normal(seed: int, name: str, n: int, device="cpu") -> torch.Tensor:
     key = _key(seed, name)
     out = torch.empty(n, dtype=torch.float32, device=device)
     scale = (1.5 ** 0.5) / 65536.0
-    for start in range(0, n, _CHUNK):
-        stop = min(n, start + _CHUNK)
+    chunk = _CHUNK_CPU if torch.device(device).type == "cpu" else _CHUNK
+    for start in range(0, n, chunk):
+        stop = min(n, start + chunk)
         i = torch.arange(start, stop, dtype=torch.int64, device=device)
         total = torch.zeros(stop - start, dtype=torch.int64, device=device)
         for word in (0, 1):

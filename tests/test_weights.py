@@ -71,7 +71,7 @@ def test_a_random_value_depends_on_seed_name_and_index_only(monkeypatch):
     assert abs(float(z.mean())) < 0.01 and abs(float(z.var()) - 1.0) < 0.01
     assert abs(float((z ** 4).mean()) - 2.85) < 0.1 and 3.5 < float(z.abs().max()) < 4.9
     # a prefix is a prefix, whatever the pieces it is drawn in
-    monkeypatch.setattr(random_init, "_CHUNK", 777)
+    monkeypatch.setattr(random_init, "_CHUNK_CPU", 777)
     assert torch.equal(standard_normal(7, name, 5000), z[:5000])
     # other seed, other name: other values, uncorrelated
     for other in (standard_normal(8, name, 200000), standard_normal(7, name + "x", 200000)):
