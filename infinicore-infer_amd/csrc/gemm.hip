@@ -415,7 +415,8 @@ static int compute_units() {
 
 // Very many weight rows and at most 16 token rows (the output head over the vocabulary): there are enough 16-row
 // weight tiles for every wave to own whole tiles, so nothing is summed across waves.  The token rows are staged in
-// LDS once per block (zero-filled beyond K; rows padded by 16 bytes so that 8 rows hit different banks); a wave
+// LDS once per block (zero-filled beyond K; rows padded by 32 bytes: the 16-byte reads of 16 rows by the 16 lanes of a
+// k-quarter then run at the full 256 bytes a cycle, with 16 bytes of padding at half of it from 8 rows on); a wave
 // walks K in groups of kWideDepth k-steps, with the next group's loads (of the same or of its next tile) issued
 // before the current group is used, so its weight stream never pauses between tiles.  A block owns a run of whole
 // tiles and its waves equal shares of the run's (tile, group) pairs, so that every wave reads the same number of
@@ -549,7 +550,7 @@ template <typename TC>
 static bool launch_gemm_wide(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
                              float alpha, const NormFuse& nf, hipStream_t stream) {
     const int steps = (K + 31) / 32, groups = (steps + kWideDepth - 1) / kWideDepth;
-    const int a_stride = groups * kWideDepth * 32 + 8;
+    const int a_stride = groups * kWideDepth * 32 + 16;
     const size_t rows_bytes = (size_t)M * a_stride * 2;
     auto lds_of = [&](int wv) { return rows_bytes + (4 * wv * 16 + 16) * sizeof(float) + (size_t)wv * 64 * 16; };
     // two blocks of 8 waves a compute unit; with many or long token rows one block of 16 waves, or of 8 when only that fits
