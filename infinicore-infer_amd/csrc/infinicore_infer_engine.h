@@ -150,10 +150,11 @@ int ic_decoder_step(IcDecoder* decoder, const IcHostBatch* batch, int* staging, 
 int ic_decoder_pack(const IcDecoder* decoder, const IcHostBatch* batch, int* staging, const int* device_ints,
                     long long n_ints, IcStepBatch* laid_out);
 
-// How many ways to split the keys of single-token rows (from sweeps on MI355X with a cold cache); see the
-// decode attention kernel.  matrix_core_head_dim: the head size when the grouped-query kernel runs, else 0.
-int ic_attn_decode_splits(int n_decode_rows, int n_kv_heads, int window, int max_context, int matrix_core_head_dim,
-                          int compute_units);
+// How many ways to split the keys of single-token rows (from sweeps on MI355X with caches that do not fit the
+// last-level cache); see the decode attention kernel.  elem_bytes: of a cache element.  matrix_cores: 1 when the
+// grouped-query kernel runs (bfloat16, several query heads per kv head).
+int ic_attn_decode_splits(int n_decode_rows, int n_kv_heads, int head_dim, int elem_bytes, int window, int max_context,
+                          int matrix_cores, int compute_units);
 
 #ifdef __cplusplus
 }

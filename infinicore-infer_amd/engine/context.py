@@ -88,6 +88,7 @@ class StepContext:
         self.max_context = 0             # most keys any single-token row sees
         self.cu_count = 256              # compute units, for split heuristics
         self.fixed_decode_splits: Optional[int] = None
+        self._splits_key, self._splits = None, 1
         self.group_views = []            # per cache group: (slots int32 [T], block tables int32 [R, max_blocks])
         self._views: Dict[int, LayerCacheView] = {}
 
@@ -97,13 +98,15 @@ class StepContext:
             v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache)
         return v
 
-    def decode_splits(self, n_kv_heads: int, window: int = 0, matrix_core_tiles_of: int = 0) -> int:
+    def decode_splits(self, n_kv_heads: int, head_dim: int, elem_bytes: int, window: int = 0, matrix_cores: bool = False) -> int:
         """How many ways to split the keys of single-token rows: the kernel library's rule
         (ic_attn_decode_splits, from sweeps on MI355X with a cold cache), so that steps issued from
-        Python and from native code split alike.  ``matrix_core_tiles_of``: the head size when the
-        grouped-query kernel runs, else 0."""
+        Python and from native code split alike.  ``matrix_cores``: the grouped-query kernel runs."""
         if self.fixed_decode_splits is not None:
             return self.fixed_decode_splits
-        from ..kernels.lib import get_lib
-        return int(get_lib().ic_attn_decode_splits(self.n_decode_rows, n_kv_heads, int(window or 0), self.max_context,
-                                                   int(matrix_core_tiles_of), self.cu_count))
+        key = (self.n_decode_rows, n_kv_heads, int(head_dim), int(elem_bytes), int(window or 0), self.max_context,
+               int(bool(matrix_cores)), self.cu_count)
+        if key != self._splits_key:             # the layers of a model mostly ask the same question
+            from ..kernels.lib import get_lib
+            self._splits_key, self._splits = key, int(get_lib().ic_attn_decode_splits(*key))
+        return self._splits

@@ -35,13 +35,17 @@ def _align4(n: int) -> int:
 
 
 def _context_bucket(n_keys: int) -> int:
-    """Key counts are rounded up to a power of two (at least 256) before the key split of
-    single-token rows is chosen, so eager and recorded steps split alike and a recorded
-    graph serves a whole range of lengths."""
+    """Key counts are rounded up before the key split of single-token rows is chosen, so eager and
+    recorded steps split alike and a recorded graph serves a whole range of lengths: to a power of
+    two up to 1,024 (at least 256), above that to a quarter of the power of two below (2,560, 3,072,
+    3,584, 4,096, 5,120 ...), so that the count the split is chosen for is at most a quarter off."""
     b = 256
     while b < n_keys:
         b *= 2
-    return b
+    if b <= 1024:
+        return b
+    q = b // 8
+    return (n_keys + q - 1) // q * q
 
 
 class _PinnedRing:
