@@ -59,14 +59,14 @@ struct IcDecoder {
     }
 
     // the last question put to ic_attn_decode_splits and its answer: the layers of a model mostly ask the same one
-    mutable int split_key[6] = {-1, -1, -1, -1, -1, -1}, split_answer = 1;
+    mutable int split_key[7] = {-1, -1, -1, -1, -1, -1, -1}, split_answer = 1;
 
     int splits_for(const IcStepBatch& b, const IcAttention& a) const {
         if (b.fixed_decode_splits > 0) return b.fixed_decode_splits;
         const int matrix_cores = (meta.dtype == IC_BF16 && a.n_heads != a.n_kv_heads) ? 1 : 0;
-        const int key[6] = {b.n_decode_rows, a.n_kv_heads, a.head_dim, a.window, b.max_context, matrix_cores};
+        const int key[7] = {b.n_decode_rows, a.n_heads, a.n_kv_heads, a.head_dim, a.window, b.max_context, matrix_cores};
         if (memcmp(key, split_key, sizeof key) != 0) {
-            split_answer = ic_attn_decode_splits(b.n_decode_rows, a.n_kv_heads, a.head_dim, dtype_size(meta.dtype), a.window,
+            split_answer = ic_attn_decode_splits(b.n_decode_rows, a.n_heads, a.n_kv_heads, a.head_dim, dtype_size(meta.dtype), a.window,
                                                  b.max_context, matrix_cores, meta.compute_units);
             memcpy(split_key, key, sizeof key);
         }
@@ -393,15 +393,30 @@ IC_EXPORT int ic_decoder_forward(IcDecoder* decoder, const IcStepBatch* batch, v
 // the full bandwidth unsplit up to 2,048 keys; many pairs want about 3.4 blocks per unit.  Grouped heads: a wave has a
 // whole 32-key tile in flight, so 128 / head size blocks per unit are enough and more only add partial results to merge.
 // A split never gets fewer than 64 keys.
-IC_EXPORT int ic_attn_decode_splits(int n_decode_rows, int n_kv_heads, int head_dim, int elem_bytes, int window, int max_context,
-                                    int matrix_cores, int compute_units) {
+IC_EXPORT int ic_attn_decode_splits(int n_decode_rows, int n_heads, int n_kv_heads, int head_dim, int elem_bytes, int window,
+                                    int max_context, int matrix_cores, int compute_units) {
     const int keys = std::max(1, window > 0 ? std::min(max_context, window) : max_context);
     const long long base = std::max(1LL, (long long)n_decode_rows * n_kv_heads);
     const double cu = compute_units > 0 ? compute_units : 256;
+    const int s_max = std::max(1, std::min(64, keys / 64));
     if (matrix_cores) {
+        // The grouped-query kernel: the same kind of model as below with constants of its own (fitted to 215 shapes of
+        // 24:8 and 16:4 heads of 64, 32:2 and 32:8 of 128, 1..64 rows, 600..16,500 keys: 1.1 % from the best count on
+        // average, worst 9 %; "128 / head size blocks a unit", which it replaces, 1.9 % and 32 %).  Up to 256 keys it
+        // does not split.
         if (keys <= 256) return 1;
-        const int want = std::max(1, (int)(128.0 / std::max(1, head_dim) * cu / (double)base + 0.5));
-        return std::max(1, std::min(std::min(want, std::max(1, keys / 64)), 64));
+        const double stream_us = (double)base * keys * std::max(1, head_dim) * 2.0 * std::max(1, elem_bytes) / (6.42e6 * cu / 256.0);
+        const double group = (double)std::max(1, n_heads) / std::max(1, n_kv_heads);
+        int best = 1;
+        double best_cost = 0.0;
+        for (int s = 1; s <= s_max; ++s) {
+            const double x = (double)base * s / cu;
+            const double lost = 1.0 + (x > 1.0 ? 0.185 : 0.801) * (std::ceil(x) / x - 1.0);
+            double cost = 1.882 + 5.201 / s + lost * stream_us;
+            if (s > 1) cost += 6.632 + 0.153 * x * group;
+            if (s == 1 || cost < best_cost) { best_cost = cost; best = s; }
+        }
+        return best;
     }
     // One head per wave: the split count with the least cost by a model of the two kernels' time in microseconds, fitted
     // to sweeps over 1..32 rows, 8..36 heads of 64 and 128, 600..16,500 keys with caches that do not fit the last-level
@@ -413,7 +428,6 @@ IC_EXPORT int ic_attn_decode_splits(int n_decode_rows, int n_kv_heads, int head_
     //   plus a start-up cost that shrinks with shorter blocks, plus, with more than one split, the second kernel, its
     //   work per split and the partial results per block.
     const double stream_us = (double)base * keys * std::max(1, head_dim) * 2.0 * std::max(1, elem_bytes) / (6.631e6 * cu / 256.0);
-    const int s_max = std::max(1, std::min(64, keys / 64));
     int best = 1;
     double best_cost = 0.0;
     for (int s = 1; s <= s_max; ++s) {

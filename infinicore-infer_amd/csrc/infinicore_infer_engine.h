@@ -153,8 +153,8 @@ int ic_decoder_pack(const IcDecoder* decoder, const IcHostBatch* batch, int* sta
 // How many ways to split the keys of single-token rows (from sweeps on MI355X with caches that do not fit the
 // last-level cache); see the decode attention kernel.  elem_bytes: of a cache element.  matrix_cores: 1 when the
 // grouped-query kernel runs (bfloat16, several query heads per kv head).
-int ic_attn_decode_splits(int n_decode_rows, int n_kv_heads, int head_dim, int elem_bytes, int window, int max_context,
-                          int matrix_cores, int compute_units);
+int ic_attn_decode_splits(int n_decode_rows, int n_heads, int n_kv_heads, int head_dim, int elem_bytes, int window,
+                          int max_context, int matrix_cores, int compute_units);
 
 #ifdef __cplusplus
 }

@@ -98,13 +98,14 @@ class StepContext:
             v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache)
         return v
 
-    def decode_splits(self, n_kv_heads: int, head_dim: int, elem_bytes: int, window: int = 0, matrix_cores: bool = False) -> int:
+    def decode_splits(self, n_heads: int, n_kv_heads: int, head_dim: int, elem_bytes: int, window: int = 0,
+                      matrix_cores: bool = False) -> int:
         """How many ways to split the keys of single-token rows: the kernel library's rule
         (ic_attn_decode_splits, from sweeps on MI355X with a cold cache), so that steps issued from
         Python and from native code split alike.  ``matrix_cores``: the grouped-query kernel runs."""
         if self.fixed_decode_splits is not None:
             return self.fixed_decode_splits
-        key = (self.n_decode_rows, n_kv_heads, int(head_dim), int(elem_bytes), int(window or 0), self.max_context,
+        key = (self.n_decode_rows, int(n_heads), n_kv_heads, int(head_dim), int(elem_bytes), int(window or 0), self.max_context,
                int(bool(matrix_cores)), self.cu_count)
         if key != self._splits_key:             # the layers of a model mostly ask the same question
             from ..kernels.lib import get_lib

@@ -78,12 +78,14 @@ class _PinnedRing:
 class Engine:
     def __init__(self, model, max_tokens: int, page_size: int = 16, max_requests: int = 64,
                  num_pages: Optional[int] = None, use_graphs: bool = True, graph_max_batch: int = 64,
-                 use_native: bool = True, max_graphs: int = 32):
+                 use_native: bool = True, max_graphs: int = 32, graph_after: int = 2):
         """``max_tokens``: the most tokens live requests hold at any time, each
         request's count rounded up to whole pages; every group's pool is sized for it.
         ``use_native``: let one native call issue a step's kernels when every part of the model
         has a native description (otherwise, and for other models, the parts' Python forward runs).
-        ``max_graphs``: recorded decode steps kept at a time (the least recently used one goes first)."""
+        ``max_graphs``: recorded decode steps kept at a time (the least recently used one goes first).
+        ``graph_after``: a decode step's shape (batch size, key-count bucket) is recorded at its n-th appearance
+        and runs eagerly before that (1: at once)."""
         self.model = model
         self.runtime: Runtime = model.runtime
         self.device = torch.device(self.runtime.device)
@@ -135,6 +137,9 @@ class Engine:
         self.graph_steps = 0         # steps that took the recorded path (the recording one included)
         self.graph_replays = 0       # of these, replays of an existing recording
         self.graphs_evicted = 0
+        self.graph_after = max(1, int(graph_after))
+        self._graph_seen: "OrderedDict[tuple, int]" = OrderedDict()     # shapes not yet recorded: how often they came
+        self.graph_deferred = 0      # decode steps run eagerly because their shape had not come back yet
         # the step function in native code, when the model's parts all have a native description
         from .native import NativeDecoder
         self.native = NativeDecoder.try_build(self) if use_native else None
@@ -459,6 +464,19 @@ class Engine:
         bucket = _context_bucket(max(starts) + 1)
         key = (R, bucket)
         g = self._graphs.get(key)
+        if g is None and self.graph_after > 1:
+            # A shape is recorded when it comes back, not when it first appears: while requests join and leave, most
+            # shapes are seen once, and recording costs several steps' time.  Until then its steps run eagerly.
+            seen = self._graph_seen.get(key, 0) + 1
+            self._graph_seen[key] = seen
+            self._graph_seen.move_to_end(key)
+            while len(self._graph_seen) > 512:
+                self._graph_seen.popitem(last=False)
+            if seen < self.graph_after:
+                self.graph_deferred += 1
+                with ops.stream_scope():
+                    return self._eager_step(entries, starts)
+            del self._graph_seen[key]
         if g is None:
             while len(self._graphs) >= self.max_graphs:          # the least recently used recording goes
                 self._graphs.popitem(last=False)

@@ -119,7 +119,7 @@ _SIGNATURES = {
     "ic_matmul_tune": [_P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _LL, _P, _LL, _I, _P],
     "ic_gemm_qkv_rope_tile_rows": [_I],
     "ic_gemm_nt_cfg": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
-    "ic_attn_decode_splits": [_I, _I, _I, _I, _I, _I, _I, _I],
+    "ic_attn_decode_splits": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
     "ic_gemm_splitk_supported": [_I, _I, _I, _I, _I],
     "ic_gemm_splitk_slices": [_I, _I],
     "ic_gemm_splitk": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P],

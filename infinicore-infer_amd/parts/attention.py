@@ -120,7 +120,7 @@ class Attention(Mixer):
                                   *args, self.scale, self.window)
             return
         if use_dec:
-            n_split = ctx.decode_splits(self.nkvh, self.dh, 2 if rt.dtype == torch.bfloat16 else 4, self.window,
+            n_split = ctx.decode_splits(self.nh, self.nkvh, self.dh, 2 if rt.dtype == torch.bfloat16 else 4, self.window,
                                         ops.attention_decode_on_matrix_cores(rt.dtype, self.nh, self.nkvh))
             part_acc = ctx.ws.buffer("attn_part_acc", (n_dec * self.nh * n_split * self.dh,), torch.float32)
             part_ml = ctx.ws.buffer("attn_part_ml", (n_dec * self.nh * n_split * 2,), torch.float32)

@@ -127,7 +127,8 @@ def test_decoding_twenty_requests_at_once(tmp_path_factory, name, dname, dtype, 
     ref = H.plain_logits(cfg, H.load_state_dict(folder), requests, dtype == torch.bfloat16)
     assert len(got) == n_req * (1 + n_dec)
     H.compare(got, ref, tol, "%s %s twenty requests" % (name, dname))
-    assert engine.graph_steps == n_dec and engine.graph_replays == n_dec - 1     # the first one records
+    # the shape runs eagerly when it first appears, is recorded when it comes back, and is replayed from then on
+    assert engine.graph_deferred == 1 and engine.graph_steps == n_dec - 1 and engine.graph_replays == n_dec - 2
     engine.cache.check_invariants()
 
 
@@ -161,7 +162,7 @@ def test_recorded_decode_steps_equal_eager_ones(tmp_path_factory, dname, dtype, 
     the replays, for two batch sizes and across a change of the key-split bucket."""
     from infinicore_infer_amd.engine import Engine, StepEntry
     folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "C")
-    a = Engine.from_dir(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4, use_graphs=True)
+    a = Engine.from_dir(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4, use_graphs=True, graph_after=1)
     b = Engine.from_dir(folder, dtype=dtype, max_tokens=1024, page_size=16, max_requests=4, use_graphs=False)
     prompts = {"p": H.random_tokens(331, 250, 1), "q": H.random_tokens(331, 40, 2), "r": H.random_tokens(331, 90, 3)}
     for eng in (a, b):
@@ -198,7 +199,7 @@ def test_recorded_steps_with_library_products_equal_eager_ones(tmp_path_factory,
     folder = os.path.join(str(tmp_path_factory.getbasetemp()), "model_%s_shaped_graph" % shape)
     write_random_model(folder, cfg, seed=11, std=0.02)
     kw = dict(dtype=torch.bfloat16, max_tokens=64 * 128, page_size=64, max_requests=65)
-    a = Engine.from_dir(folder, use_graphs=True, **kw)
+    a = Engine.from_dir(folder, use_graphs=True, graph_after=1, **kw)
     b = Engine.from_dir(folder, use_graphs=False, **kw)
     if shape == "2b":                        # with the algorithms that timing chooses for these row counts (kept per process)
         a.tune_library_products([64, 20])
@@ -351,7 +352,30 @@ def test_benchmark_shaped_layers(tmp_path_factory):
     for (rid, pos), row in got.items():
         err = float((row.double() - ref[rid][pos]).abs().max()) / scale
         assert err <= H.BF16_TOL, "request %s position %d differs by %.3g of the largest logit" % (rid, pos, err)
-    assert engine.graph_steps >= 9
+    assert engine.graph_steps + engine.graph_deferred >= 9 and engine.graph_replays >= 6
+
+
+def test_a_shape_is_recorded_when_it_comes_back(tmp_path_factory):
+    """While requests join and leave, most decode shapes (batch size, key-count bucket) are seen once: such a step runs
+    eagerly.  A shape that comes back is recorded then and replayed afterwards.  All three ways give the same bits."""
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    cfg = H.CONFIGS["A"][0]
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "A")
+    a = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=512, page_size=16, max_requests=4)
+    b = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=512, page_size=16, max_requests=4, use_graphs=False)
+    assert a.graph_after == 2
+    ids = ["x", "y", "z"]
+    for eng in (a, b):
+        eng.step([StepEntry(r, H.random_tokens(cfg["vocab_size"], 5 + 3 * i, i), []) for i, r in enumerate(ids)])
+    toks = H.random_tokens(cfg["vocab_size"], 40, 8)
+    seen = []
+    for i, n in enumerate([3, 2, 1, 3, 3, 2, 3, 1, 1]):          # batch sizes as requests pause and resume
+        ents = [StepEntry(r, [toks[i + j]], [0]) for j, r in enumerate(ids[:n])]
+        assert torch.equal(a.step(ents).clone(), b.step(ents).clone()), "step %d" % i
+        seen.append((a.graph_deferred, a.graph_steps, a.graph_replays, len(a._graphs)))
+    # sizes 3, 2, 1 first run eagerly; the second 3 records, the third replays; the second 2 records; ...
+    assert seen[2] == (3, 0, 0, 0) and seen[3] == (3, 1, 0, 1) and seen[4] == (3, 2, 1, 1)
+    assert seen[5] == (3, 3, 1, 2) and seen[6] == (3, 4, 2, 2) and seen[7] == (3, 5, 2, 3) and seen[8] == (3, 6, 3, 3)
 
 
 @pytest.mark.parametrize("native", [True, False])
@@ -363,7 +387,7 @@ def test_recorded_steps_hold_a_bounded_amount_of_memory(tmp_path_factory, native
     cfg = H.CONFIGS["C"][0]
     folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "C")
     eng = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=64 * 64, page_size=16, max_requests=64,
-                          max_graphs=12, use_native=native)
+                          max_graphs=12, use_native=native, graph_after=1)
     ids = ["g%d" % i for i in range(64)]
     eng.step([StepEntry(r, H.random_tokens(cfg["vocab_size"], 3 + i % 9, i), []) for i, r in enumerate(ids)])
     sizes = []
