@@ -345,8 +345,9 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
         ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15) || ((uintptr_t)tiles & 15)) return IC_ERR_ARG;
     const float sl2 = scale * 1.4426950408889634f;
     const bool staged = bt_stride <= kPfMaxPages;       // a block never needs more page ids than a request has
-    // Few blocks (under 2.75 per compute unit, measured): the longest tile's walk over the keys sets the
-    // time, so two wave groups share it.  Many blocks: one group, more blocks resident.
+    // Few blocks (up to 2 per compute unit; measured with 16..64 heads of 64 and 32..40 of 128 over 512..4,096
+    // tokens: two groups win up to 2.0 blocks a unit by 5..25 %, one group from 2.25 on by 2..25 %): the longest
+    // tile's walk over the keys sets the time, so two wave groups share it.  Many blocks: one group, more blocks resident.
     static int cus = 0;                                 // compute units of the device, asked once
     if (cus == 0) {
         int dev = 0, n = 0;
@@ -354,7 +355,7 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
             hipDeviceGetAttribute(&n, hipDeviceAttributeMultiprocessorCount, dev) == hipSuccess && n > 0) cus = n;
         else cus = 256;
     }
-    const bool two_groups = groups ? groups == 2 : 4LL * nh * n_tiles < 11LL * cus;
+    const bool two_groups = groups ? groups == 2 : (long long)nh * n_tiles <= 2LL * cus;
     dim3 grid((unsigned)nh * (unsigned)n_tiles);
     const bool page64 = page_size >= kPfKeys;            // (a power of two) a 64-key tile lies in one page
 #define IC_PF_LAUNCH(DD, ST, GG, PP)                                                                                   \
