@@ -36,12 +36,15 @@ class GroupSpec:
     head_dim: int
     window: Optional[int] = None
     slots: tuple = ()                   # cache slot ids (positions in the model's cache list)
+    planes: int = 2                     # tensors per slot (keys and values: 2; one latent per token: 1)
 
     def __post_init__(self):
         if self.kind not in ("full", "window"):
             raise CacheError("group kind must be 'full' or 'window'")
         if self.kind == "window" and not (self.window and self.window > 0):
             raise CacheError("a window group needs a positive window")
+        if self.planes <= 0:
+            raise CacheError("a group needs at least one plane")
 
 
 class PagePool:

@@ -1,10 +1,11 @@
 """Device memory of the cache: the page planes of each group and the
 per-request state tensors.
 
-Layout of one cache slot (one attention layer's keys or values):
+Layout of one plane of a cache slot (one attention layer's keys or values):
 ``[num_pages, n_kv_heads, page_size, head_dim]``: the keys of one head inside a
 page are one contiguous run, which is what the attention kernels stream.
-A group holds ``[n_slots, 2 (K, V), num_pages, n_kv_heads, page_size, head_dim]``.
+A group holds ``[n_slots, planes, num_pages, n_kv_heads, page_size, head_dim]``;
+attention has two planes (K, V), a mixer that caches one vector per token has one.
 """
 from typing import Dict, List, Sequence, Tuple
 
@@ -22,7 +23,7 @@ class CacheStorage:
         self.group_planes: List[torch.Tensor] = []
         self._slot_index: Dict[int, Tuple[int, int]] = {}      # cache slot -> (group, index in group)
         for g, spec in enumerate(groups):
-            planes = torch.empty((len(spec.slots), 2, num_pages[g], spec.n_kv_heads, page_size, spec.head_dim),
+            planes = torch.empty((len(spec.slots), spec.planes, num_pages[g], spec.n_kv_heads, page_size, spec.head_dim),
                                  dtype=dtype, device=device)
             self.group_planes.append(planes)
             for i, s in enumerate(spec.slots):
@@ -38,16 +39,24 @@ class CacheStorage:
     def group_of(self, slot: int) -> int:
         return self._slot_index[slot][0]
 
-    def kv(self, slot: int):
-        """(K plane, V plane) of a cache slot (views made once: the planes never move)."""
-        kv = self._kv_views.get(slot)
-        if kv is None:
+    def planes(self, slot: int) -> tuple:
+        """The planes of a cache slot, each [num_pages, n_kv_heads, page_size, head_dim] (views made
+        once: the planes never move)."""
+        views = self._kv_views.get(slot)
+        if views is None:
             g, i = self._slot_index[slot]
-            kv = self._kv_views[slot] = (self.group_planes[g][i, 0], self.group_planes[g][i, 1])
-        return kv
+            views = self._kv_views[slot] = tuple(self.group_planes[g][i, j] for j in range(self.group_planes[g].shape[1]))
+        return views
+
+    def kv(self, slot: int):
+        """(K plane, V plane) of a cache slot with two planes."""
+        views = self.planes(slot)
+        if len(views) != 2:
+            raise ValueError("cache slot %d has %d planes, not keys and values" % (slot, len(views)))
+        return views
 
     def copy_pages(self, group: int, src_pages: Sequence[int], dst_pages: Sequence[int]) -> None:
-        """Copy whole pages inside a group: every cache slot of the group, keys and values."""
+        """Copy whole pages inside a group: every cache slot of the group, every plane."""
         if not src_pages:
             return
         from ..kernels import ops

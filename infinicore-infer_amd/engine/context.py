@@ -48,13 +48,20 @@ class Workspace:
 
 @dataclass
 class LayerCacheView:
-    """What a mixer sees of its cache slot in this step."""
-    k: Optional[torch.Tensor] = None             # [pages, kv_heads, page_size, head_dim]
-    v: Optional[torch.Tensor] = None
+    """What a mixer sees of its cache slot in this step: the planes of its paged memory (if it asked for
+    any) with the step's token slots and block tables, and its fixed-size state (if it asked for one)."""
+    k: Optional[torch.Tensor] = None             # plane 0 [pages, kv_heads, page_size, head_dim]
+    v: Optional[torch.Tensor] = None             # plane 1 (None for a slot with one plane)
     slots: Optional[torch.Tensor] = None         # int32 [T]: token slot of each new token in this group
     block_tables: Optional[torch.Tensor] = None  # int32 [R, max_blocks]
     state: Optional[torch.Tensor] = None         # [max_requests, ...] fixed-size state of this slot
     writes: bool = True
+    planes: tuple = ()                           # every plane of the slot, in order (k and v are the first two)
+
+    @classmethod
+    def of_planes(cls, planes, slots, block_tables, state=None) -> "LayerCacheView":
+        return cls(k=planes[0], v=planes[1] if len(planes) > 1 else None, slots=slots, block_tables=block_tables,
+                   state=state, planes=tuple(planes))
 
 
 class StepContext:
@@ -73,6 +80,7 @@ class StepContext:
         self.want_rows = None            # int32 [W]  token rows whose logits are wanted
         self.n_want = 0
         self.want_rows_identity = False  # every row's logits are wanted, in order
+        # listed when some part of the model asks for them (Part.portion_tile_rows):
         self.decode_rows = None          # int32 [n_decode_rows] rows that are a request's single token
         self.n_decode_rows = 0
         self.decode_rows_identity = False
@@ -86,28 +94,14 @@ class StepContext:
         self.host_state_slots: List[int] = []
         self.max_position = 0            # largest position in the step
         self.max_context = 0             # most keys any single-token row sees
-        self.cu_count = 256              # compute units, for split heuristics
-        self.fixed_decode_splits: Optional[int] = None
-        self._splits_key, self._splits = None, 1
+        self.cu_count = 256              # compute units of the device, for the parts' launch heuristics
+        self.fixed_decode_splits: Optional[int] = None   # a recorded step's fixed way of splitting single-token rows' keys
+        self.memo: Dict[str, object] = {}  # scratch of the parts for this step (what several layers would work out alike)
         self.group_views = []            # per cache group: (slots int32 [T], block tables int32 [R, max_blocks])
         self._views: Dict[int, LayerCacheView] = {}
 
     def cache_view(self, entry) -> LayerCacheView:
         v = self._views[entry.cache]
         if v.writes != entry.writes_cache:
-            v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache)
+            v = LayerCacheView(v.k, v.v, v.slots, v.block_tables, v.state, entry.writes_cache, v.planes)
         return v
-
-    def decode_splits(self, n_heads: int, n_kv_heads: int, head_dim: int, elem_bytes: int, window: int = 0,
-                      matrix_cores: bool = False) -> int:
-        """How many ways to split the keys of single-token rows: the kernel library's rule
-        (ic_attn_decode_splits, from sweeps on MI355X with a cold cache), so that steps issued from
-        Python and from native code split alike.  ``matrix_cores``: the grouped-query kernel runs."""
-        if self.fixed_decode_splits is not None:
-            return self.fixed_decode_splits
-        key = (self.n_decode_rows, int(n_heads), n_kv_heads, int(head_dim), int(elem_bytes), int(window or 0), self.max_context,
-               int(bool(matrix_cores)), self.cu_count)
-        if key != self._splits_key:             # the layers of a model mostly ask the same question
-            from ..kernels.lib import get_lib
-            self._splits_key, self._splits = key, int(get_lib().ic_attn_decode_splits(*key))
-        return self._splits

@@ -103,11 +103,11 @@ class Engine:
         needs = model.cache_needs()
         keyed: Dict[tuple, List[int]] = {}
         for slot, need in enumerate(needs):
-            if need.kind == "kv":
-                keyed.setdefault((need.n_kv_heads, need.head_dim, need.window), []).append(slot)
+            if need.paged:
+                keyed.setdefault((need.planes, need.n_kv_heads, need.head_dim, need.window), []).append(slot)
         self.groups: List[GroupSpec] = [
-            GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots))
-            for (nkv, dh, w), slots in keyed.items()]
+            GroupSpec("window" if w else "full", nkv, dh, w, tuple(slots), planes)
+            for (planes, nkv, dh, w), slots in keyed.items()]
         # positions a request may reach: the model's limit and that of every part (a table's length)
         limits = [model.spec.max_positions] + [p.position_limit() for p in model.all_parts()]
         self.max_positions = min(int(l) for l in limits if l is not None)
@@ -116,7 +116,7 @@ class Engine:
         self.storage = CacheStorage(self.groups, [self.num_pages] * len(self.groups), self.page_size,
                                     self.runtime.dtype, self.device)
         for slot, need in enumerate(needs):
-            if need.kind == "state":
+            if need.has_state:
                 self.storage.add_state(slot, self.max_requests, need.state_shape, need.state_dtype)
         self._slot_group = {s: g for g, spec in enumerate(self.groups) for s in spec.slots}
         self.has_state = bool(self.storage.state)      # some mixer keeps fixed-size state per request
@@ -125,7 +125,11 @@ class Engine:
         self.ws = Workspace(self.device)
         self._ring = _PinnedRing()
         self._meta_dev: Optional[torch.Tensor] = None
-        self._tile_rows = ops.attention_prefill_tile_rows()
+        # tiles of prompt portions and rows of single tokens are listed for the parts that ask for them
+        tile_rows = {int(r) for r in (p.portion_tile_rows() for p in model.all_parts()) if r}
+        if len(tile_rows) > 1:
+            raise ValueError("parts of the model ask for prompt tiles of different heights: %s" % sorted(tile_rows))
+        self._tile_rows = tile_rows.pop() if tile_rows else 0
         self.cu_count = torch.cuda.get_device_properties(self.device).multi_processor_count
         self.steps_run = 0
         # decode steps (one token per request, its logits wanted) replay a captured HIP graph
@@ -362,8 +366,11 @@ class Engine:
             row0 = req_start[r]
             want_rows.extend(row0 + int(w) for w in e.want)
             if n == 1:
-                decode_rows.append((p0, row0))
                 max_ctx = max(max_ctx, p0 + 1)
+            if not self._tile_rows:
+                continue
+            if n == 1:
+                decode_rows.append((p0, row0))
             else:
                 for o in range(0, n, self._tile_rows):
                     tiles.append((r, row0 + o, min(self._tile_rows, n - o), p0 + o))
@@ -432,7 +439,7 @@ class Engine:
         ctx.want_rows, ctx.n_want = view("want_rows"), len(want_rows)
         ctx.want_rows_identity = (len(want_rows) == T and all(w == i for i, w in enumerate(want_rows)))
         ctx.decode_rows, ctx.n_decode_rows = view("decode_rows"), len(decode_rows)
-        ctx.decode_rows_identity = (len(decode_rows) == T)
+        ctx.decode_rows_identity = (len(decode_rows) == T and T > 0)
         ctx.prefill_tiles = view("tiles").view(-1, 4)
         ctx.n_prefill_tiles = len(tiles)
         ctx.req_start, ctx.req_pos = req_start, list(starts)
@@ -445,12 +452,12 @@ class Engine:
         group_views = [(view("slots%d" % g), view("tables%d" % g).view(R, group_maxb[g])) for g in range(n_groups)]
         ctx.group_views = group_views
         for slot in range(self.model.spec.num_cache_slots()):
+            state = self.storage.state.get(slot)
             if slot in self._slot_group:
                 slots, tables_g = group_views[self._slot_group[slot]]
-                k, v = self.storage.kv(slot)
-                ctx._views[slot] = LayerCacheView(k=k, v=v, slots=slots, block_tables=tables_g)
+                ctx._views[slot] = LayerCacheView.of_planes(self.storage.planes(slot), slots, tables_g, state)
             else:
-                ctx._views[slot] = LayerCacheView(state=self.storage.state.get(slot))
+                ctx._views[slot] = LayerCacheView(state=state)
         return ctx
 
     # ---- decode steps as captured graphs ------------------------------------------------------------
@@ -613,13 +620,13 @@ class _DecodeGraph:
         ctx.cu_count = engine.cu_count
         ctx.group_views = [(view("slots%d" % g), view("tables%d" % g).view(R, self.maxb)) for g in range(ng)]
         for slot in range(engine.model.spec.num_cache_slots()):
+            state = engine.storage.state.get(slot)
             if slot in engine._slot_group:
                 g = engine._slot_group[slot]
-                k, v = engine.storage.kv(slot)
-                ctx._views[slot] = LayerCacheView(k=k, v=v, slots=view("slots%d" % g),
-                                                  block_tables=view("tables%d" % g).view(R, self.maxb))
+                ctx._views[slot] = LayerCacheView.of_planes(engine.storage.planes(slot), view("slots%d" % g),
+                                                            view("tables%d" % g).view(R, self.maxb), state)
             else:
-                ctx._views[slot] = LayerCacheView(state=engine.storage.state.get(slot))
+                ctx._views[slot] = LayerCacheView(state=state)
         self.ctx = ctx
 
     def fill(self, engine, entries, starts):

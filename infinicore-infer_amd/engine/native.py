@@ -49,8 +49,9 @@ class NativeDecoder:
         layers = [l.native_desc() for l in model.layers]
         if emb is None or head is None or not isinstance(fin, IcNorm) or not all(isinstance(l, IcLayer) for l in layers):
             return None
-        if any(s not in engine._slot_group for s in range(model.spec.num_cache_slots())):
-            return None                   # a slot of fixed-size state: no built-in part has one
+        if engine.has_state or any(g.planes != 2 for g in engine.groups) or \
+                any(s not in engine._slot_group for s in range(model.spec.num_cache_slots())):
+            return None                   # fixed-size state or a cache that is not keys and values: no built-in part has one
         scaled = model.head.deferred_norm(model.final_norm)
         if scaled is None:
             return None

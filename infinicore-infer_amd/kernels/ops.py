@@ -207,6 +207,15 @@ def attention_decode_on_matrix_cores(dtype, n_heads: int, n_kv_heads: int) -> bo
     return dtype == torch.bfloat16 and n_heads != n_kv_heads
 
 
+def attention_decode_splits(n_rows: int, n_heads: int, n_kv_heads: int, head_dim: int, elem_bytes: int, window: int,
+                            max_context: int, matrix_cores: int, compute_units: int) -> int:
+    """Ways to split the keys of ``n_rows`` single-token rows that see up to ``max_context`` keys (the library's
+    cost model of its two kernels, fitted to sweeps)."""
+    return int(get_lib().ic_attn_decode_splits(int(n_rows), int(n_heads), int(n_kv_heads), int(head_dim), int(elem_bytes),
+                                               int(window or 0), int(max_context), int(bool(matrix_cores)),
+                                               int(compute_units)))
+
+
 def attention_decode(q, out, kcache, vcache, block_tables, tok_list, n_tok, token_req, positions, part_acc,
                      part_ml, n_heads, n_kv_heads, head_dim, page_size, scale: float, window: int, n_split: int):
     """Split-key attention of the single tokens listed in tok_list (None: rows 0..n_tok-1)."""

@@ -49,6 +49,9 @@ class Attention(Mixer):
     def cache_need(self):
         return CacheNeed("kv", self.nkvh, self.dh, self.window or None)
 
+    def portion_tile_rows(self):
+        return ops.attention_prefill_tile_rows()
+
     # ---- weights: names of scripts/jiuge.py:45-63 ------------------------------
     def weight_specs(self):
         n = self.name
@@ -106,6 +109,21 @@ class Attention(Mixer):
         linear(out, self.w_o, y, rt.gemm_impl)
         return y
 
+    def _key_splits(self, ctx) -> int:
+        """How many ways to split the keys of single-token rows: the kernel library's rule
+        (ic_attn_decode_splits, from sweeps on MI355X with a cold cache), so that steps issued from
+        Python and from native code split alike.  The layers of a model mostly ask the same question,
+        so the answer is kept in the step's memo."""
+        if ctx.fixed_decode_splits is not None:
+            return ctx.fixed_decode_splits
+        rt = self.runtime
+        key = (ctx.n_decode_rows, self.nh, self.nkvh, self.dh, 2 if rt.dtype == torch.bfloat16 else 4, self.window,
+               ctx.max_context, int(ops.attention_decode_on_matrix_cores(rt.dtype, self.nh, self.nkvh)), ctx.cu_count)
+        memo = ctx.memo.get("attention_key_splits")
+        if memo is None or memo[0] != key:
+            memo = ctx.memo["attention_key_splits"] = (key, ops.attention_decode_splits(*key))
+        return memo[1]
+
     def _attend(self, q, out, ctx, cache):
         rt = self.runtime
         args = (self.nh, self.nkvh, self.dh, ctx.page_size)
@@ -120,8 +138,7 @@ class Attention(Mixer):
                                   *args, self.scale, self.window)
             return
         if use_dec:
-            n_split = ctx.decode_splits(self.nh, self.nkvh, self.dh, 2 if rt.dtype == torch.bfloat16 else 4, self.window,
-                                        ops.attention_decode_on_matrix_cores(rt.dtype, self.nh, self.nkvh))
+            n_split = self._key_splits(ctx)
             part_acc = ctx.ws.buffer("attn_part_acc", (n_dec * self.nh * n_split * self.dh,), torch.float32)
             part_ml = ctx.ws.buffer("attn_part_ml", (n_dec * self.nh * n_split * 2,), torch.float32)
             ops.attention_decode(q, out, cache.k, cache.v, cache.block_tables,

@@ -31,8 +31,11 @@ class Runtime:
 @dataclass(frozen=True)
 class CacheNeed:
     """What a mixer needs from the cache manager.
-    kind 'kv': paged keys and values of n_kv_heads x head_dim, all of them or a window;
+    kind 'kv': paged memory, ``planes`` tensors per cache slot that hold ``n_kv_heads`` rows of
+    ``head_dim`` values for every token (keys and values of attention: 2 planes; one latent vector
+    per token: planes = 1, n_kv_heads = 1, head_dim = its width), all tokens or a window of them;
     kind 'state': a fixed-size tensor of ``state_shape`` per request;
+    kind 'kv+state': both, for a mixer that walks a paged cache and carries a running state as well;
     kind 'none': nothing."""
     kind: str = "none"
     n_kv_heads: int = 0
@@ -40,6 +43,24 @@ class CacheNeed:
     window: Optional[int] = None
     state_shape: Tuple[int, ...] = ()
     state_dtype: torch.dtype = torch.float32
+    planes: int = 2
+
+    def __post_init__(self):
+        if self.kind not in ("none", "kv", "state", "kv+state"):
+            raise ValueError("cache need of kind %r (have none, kv, state, kv+state)" % (self.kind,))
+        if self.paged and (self.n_kv_heads <= 0 or self.head_dim <= 0 or self.planes <= 0):
+            raise ValueError("a paged cache need names planes, rows per token and their width (got %d, %d, %d)"
+                             % (self.planes, self.n_kv_heads, self.head_dim))
+        if self.has_state and not self.state_shape:
+            raise ValueError("a state need names the state's shape")
+
+    @property
+    def paged(self) -> bool:
+        return self.kind in ("kv", "kv+state")
+
+    @property
+    def has_state(self) -> bool:
+        return self.kind in ("state", "kv+state")
 
 
 @dataclass
@@ -149,6 +170,12 @@ class Part:
     def _forward_is(self, cls) -> bool:
         """True when this object's forward is ``cls``'s own (no subclass changed what a step does)."""
         return type(self).forward is cls.forward
+
+    def portion_tile_rows(self):
+        """Rows per tile when this part wants the step's batch listed as tiles of prompt portions and
+        rows of single tokens (``StepContext.prefill_tiles`` and ``decode_rows``), else None.  Parts of
+        one model that ask must ask for the same tile height."""
+        return None
 
     def position_limit(self):
         """Positions this part can take (a table's length), or None when it has no limit.  The

@@ -59,11 +59,12 @@ class DecoderModel:
                 continue
             wn = self.layers[writers[e.cache]].mixer.cache_need()
             rn = self.layers[e.layer].mixer.cache_need()
-            if wn.kind != "kv" or rn.kind != "kv":
+            if not (wn.paged and rn.paged):
                 continue
-            if (rn.n_kv_heads, rn.head_dim) != (wn.n_kv_heads, wn.head_dim):
-                raise ValueError("layer %d reads cache slot %d with %d kv heads of %d, its writer (layer %d) keeps %d of %d"
-                                 % (e.layer, e.cache, rn.n_kv_heads, rn.head_dim, writers[e.cache], wn.n_kv_heads, wn.head_dim))
+            if (rn.planes, rn.n_kv_heads, rn.head_dim) != (wn.planes, wn.n_kv_heads, wn.head_dim):
+                raise ValueError("layer %d reads cache slot %d as %d planes with %d kv heads of %d, its writer (layer %d) "
+                                 "keeps %d planes with %d of %d" % (e.layer, e.cache, rn.planes, rn.n_kv_heads, rn.head_dim,
+                                                                    writers[e.cache], wn.planes, wn.n_kv_heads, wn.head_dim))
             if wn.window and (not rn.window or rn.window > wn.window):
                 raise ValueError("layer %d reads cache slot %d over %s keys, its writer (layer %d) keeps a window of %d"
                                  % (e.layer, e.cache, rn.window or "all", writers[e.cache], wn.window))

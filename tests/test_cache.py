@@ -162,3 +162,29 @@ def test_fork_copies_the_first_tokens_into_pages_of_its_own():
     m.release("a")
     m.append("b", 20)                              # the copy goes on by itself
     m.check_invariants()
+
+
+def test_a_cache_need_names_planes_pages_and_state_together():
+    """A mixer may ask for paged memory of any number of planes, for a fixed-size state, or for both."""
+    import torch
+    from infinicore_infer_amd.cache import CacheStorage
+    from infinicore_infer_amd.parts import CacheNeed
+    kv = CacheNeed("kv", 2, 16)
+    assert kv.paged and not kv.has_state and kv.planes == 2
+    latent = CacheNeed("kv+state", n_kv_heads=1, head_dim=24, planes=1, state_shape=(5,))
+    assert latent.paged and latent.has_state
+    assert CacheNeed("state", state_shape=(3, 2)).has_state and not CacheNeed("state", state_shape=(3,)).paged
+    assert not CacheNeed().paged and not CacheNeed().has_state
+    for bad in (dict(kind="pages"), dict(kind="kv", n_kv_heads=0, head_dim=8), dict(kind="kv", n_kv_heads=1, head_dim=8, planes=0),
+                dict(kind="state"), dict(kind="kv+state", n_kv_heads=1, head_dim=8)):
+        with pytest.raises(ValueError):
+            CacheNeed(**bad)
+    with pytest.raises(CacheError):
+        GroupSpec("full", 1, 8, planes=0)
+    groups = [GroupSpec("full", 1, 24, None, (0, 2), planes=1), GroupSpec("full", 2, 16, None, (1,))]
+    st = CacheStorage(groups, [3, 3], 4, torch.float32, "cpu")
+    assert tuple(st.group_planes[0].shape) == (2, 1, 3, 1, 4, 24) and tuple(st.group_planes[1].shape) == (1, 2, 3, 2, 4, 16)
+    assert len(st.planes(2)) == 1 and len(st.planes(1)) == 2 and len(st.kv(1)) == 2
+    assert st.planes(2)[0].data_ptr() == st.group_planes[0][1, 0].data_ptr()
+    with pytest.raises(ValueError):
+        st.kv(0)

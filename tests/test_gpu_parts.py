@@ -551,3 +551,156 @@ def test_toy_architecture_with_routed_experts_and_another_position_encoding():
         got = H.run_trace(eng, steps)
         H.compare(got, ref, 2e-4, "toy routed %s" % maker.__name__)
         eng.cache.check_invariants()
+
+
+# ---------------------------------------------------------------------------
+# a third toy architecture: a mixer that caches ONE latent vector per token in pages (one plane,
+# no keys and values, no heads) and carries a running state per request beside it
+# ---------------------------------------------------------------------------
+def _register_toy_latent():
+    from infinicore_infer_amd.config import LayerSpec, ModelSpec, PartSpec, default_schedule, register_architecture
+    from infinicore_infer_amd.parts import CacheNeed, Mixer, register_part
+    from infinicore_infer_amd.weights import WeightSpec
+
+    @register_part("mixer", "toy_latent_memory")
+    class LatentMemory(Mixer):
+        """c_t = W_down h_t is cached; y_t = W_up (sum_s softmax_s(c_t . c_s / sqrt(L)) c_s + mean_{s <= t} c_s),
+        s over the tokens up to t.  The softmax walks the paged latents, the mean comes from a running
+        sum and count kept as the request's state."""
+
+        def __init__(self, name, runtime, hidden_size, latent_size):
+            super().__init__(name, runtime)
+            self.d, self.L = hidden_size, latent_size
+
+        def cache_need(self):
+            return CacheNeed("kv+state", n_kv_heads=1, head_dim=self.L, planes=1, state_shape=(self.L + 1,),
+                             state_dtype=torch.float32)
+
+        def weight_specs(self):
+            return {self.name + "down.weight": WeightSpec((self.L, self.d)), self.name + "up.weight": WeightSpec((self.d, self.L))}
+
+        def load_weights(self, tensors):
+            self.w_down, self.w_up = tensors[self.name + "down.weight"], tensors[self.name + "up.weight"]
+
+        def forward(self, h, ctx, cache):
+            assert len(cache.planes) == 1 and cache.v is None and cache.state is not None
+            ps = ctx.page_size
+            c = (h @ self.w_down.t()).float()
+            latents = cache.planes[0].view(-1, self.L)               # [pages * page_size, L]: one row per token slot
+            if cache.writes:
+                latents[cache.slots.long()] = c.to(latents.dtype)
+            y = ctx.ws.buffer("toy_latent_out", tuple(h.shape), self.runtime.dtype)
+            for r in range(ctx.R):
+                a, b, p0 = ctx.req_start[r], ctx.req_start[r + 1], ctx.req_pos[r]
+                pos = torch.arange(p0 + b - a, device=h.device)
+                mem = latents[cache.block_tables[r].long()[pos // ps] * ps + pos % ps].float()       # every latent so far
+                scores = c[a:b] @ mem.t() / self.L ** 0.5
+                scores = scores.masked_fill(pos[None, :] > pos[p0:, None], float("-inf"))
+                st = cache.state[ctx.host_state_slots[r]]
+                run = torch.cumsum(c[a:b], 0) + st[:-1]
+                n = st[-1] + torch.arange(1, b - a + 1, device=h.device)
+                y[a:b] = ((torch.softmax(scores, -1) @ mem + run / n[:, None]) @ self.w_up.float().t()).to(y.dtype)
+                st[:-1] = run[-1]
+                st[-1] = n[-1]
+            return y
+
+    class LatentConfig:
+        def __init__(self, cfg):
+            self.cfg = cfg
+
+        @classmethod
+        def from_dict(cls, cfg, **kw):
+            return cls(cfg)
+
+        def model_spec(self):
+            c = self.cfg
+            d, nh, dh = c["hidden"], c["heads"], c["head_dim"]
+            rot = PartSpec("rotary", "", {"head_dim": dh, "theta": 500.0, "max_positions": c["max_pos"]})
+            norm = lambda p: PartSpec("rmsnorm", p, {"size": d, "eps": 1e-5})
+            layers = []
+            for i in range(3):
+                p = "layers.%d." % i
+                mixer = PartSpec("toy_latent_memory", p + "mem.", {"hidden_size": d, "latent_size": c["latent"]}) if i != 1 else \
+                    PartSpec("attention", p + "att.", {"hidden_size": d, "num_heads": nh, "num_kv_heads": 1, "head_dim": dh,
+                                                       "softmax_scale": dh ** -0.5, "position_encoding": rot})
+                layers.append(LayerSpec(PartSpec("prenorm_residual", p, {"residual_scale": 0.7}), mixer, norm(p + "n1."),
+                                        PartSpec("swiglu", p + "mlp.", {"hidden_size": d, "intermediate_size": c["inner"]}),
+                                        norm(p + "n2.")))
+            return ModelSpec("toy-latent", c["vocab"], d, c["max_pos"],
+                             PartSpec("embedding", "emb.", {"vocab_size": c["vocab"], "hidden_size": d, "scale": 1.0}),
+                             layers, default_schedule(3), norm("final."),
+                             PartSpec("lm_head", "head.", {"vocab_size": c["vocab"], "hidden_size": d, "logit_scale": 1.0}))
+
+    register_architecture(["toy-latent-arch"], LatentConfig)
+
+
+def _toy_latent_plain(model, cfg, tokens):
+    T, nh, dh, L = len(tokens), cfg["heads"], cfg["head_dim"], cfg["latent"]
+    half = dh // 2
+    cpu = lambda t: t.detach().cpu().double()
+    sin, cos = P.plain_rope_tables(dh, 500.0, T)
+
+    def rope(x):
+        s, c = sin[:T, None, :], cos[:T, None, :]
+        return torch.cat([x[..., :half] * c - x[..., half:] * s, x[..., :half] * s + x[..., half:] * c], -1)
+
+    causal = torch.tril(torch.ones(T, T, dtype=torch.bool))
+    x = P.plain_embedding(cpu(model.embedding.table), tokens, 1.0)
+    for blk in model.layers:
+        h = P.plain_rmsnorm(x, cpu(blk.mixer_norm.weight), 1e-5)
+        m = blk.mixer
+        if hasattr(m, "w_down"):
+            c = P.plain_linear(h, cpu(m.w_down))
+            p = torch.softmax((c @ c.t() / L ** 0.5).masked_fill(~causal, float("-inf")), -1)
+            mean = torch.cumsum(c, 0) / torch.arange(1, T + 1)[:, None]
+            y = P.plain_linear(p @ c + mean, cpu(m.w_up))
+        else:
+            qkv = P.plain_linear(h, cpu(m.w_qkv))
+            q = rope(qkv[:, :nh * dh].reshape(T, nh, dh))
+            k = rope(qkv[:, nh * dh:(nh + 1) * dh].reshape(T, 1, dh))
+            v = qkv[:, (nh + 1) * dh:].reshape(T, 1, dh)
+            y = P.plain_linear(P.plain_attention(q, k, v, dh ** -0.5, 0, None).reshape(T, nh * dh), cpu(m.w_o))
+        x = x + 0.7 * y
+        h = P.plain_rmsnorm(x, cpu(blk.feed_forward_norm.weight), 1e-5)
+        gu = P.plain_linear(h, cpu(blk.feed_forward.w_gate_up))
+        di = gu.shape[1] // 2
+        x = x + 0.7 * P.plain_linear(P.plain_swiglu(gu[:, :di], gu[:, di:]), cpu(blk.feed_forward.w_down))
+    return P.plain_linear(P.plain_rmsnorm(x, cpu(model.final_norm.weight), 1e-5), cpu(model.head.weight))
+
+
+def test_toy_architecture_with_a_one_plane_latent_cache_and_a_state_in_one_mixer():
+    """A mixer that asks for paged memory of one plane (a latent vector per token) AND a fixed-size state,
+    beside the package's attention with its keys and values: two cache groups of different plane counts,
+    pages given back and used again, a forked request, no change to the framework's files."""
+    from infinicore_infer_amd.config import config_from_dict
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    from infinicore_infer_amd.parts import Runtime, build_model
+    from infinicore_infer_amd.weights import init_random_weights
+    _register_toy_latent()
+    cfg = {"model_type": "toy-latent-arch", "vocab": 83, "hidden": 56, "heads": 3, "head_dim": 32, "latent": 24, "inner": 72,
+           "max_pos": 192}
+    model = build_model(config_from_dict(cfg).model_spec(), Runtime(torch.float32, DEV))
+    init_random_weights(model, seed=23, std=0.2, norm_std=0.1, tie=False)
+    needs = model.cache_needs()
+    assert [(n.kind, n.planes if n.paged else 0) for n in needs] == [("kv+state", 1), ("kv", 2), ("kv+state", 1)]
+    requests = {"z%d" % i: H.random_tokens(83, n, 80 + i) for i, n in enumerate([66, 21, 110, 5])}
+    ref = {rid: _toy_latent_plain(model, cfg, toks) for rid, toks in requests.items()}
+    for maker in (H.trace_whole, H.trace_chunks, H.trace_mixed):
+        steps, max_tokens = maker(requests)
+        eng = Engine(model, max_tokens=max_tokens, page_size=16, max_requests=4)
+        assert sorted((g.planes, g.n_kv_heads, g.head_dim, len(g.slots)) for g in eng.groups) == [(1, 1, 24, 2), (2, 1, 32, 1)]
+        assert eng.native is None and not eng.use_graphs and eng.has_state
+        assert [tuple(p.shape[:2]) for p in eng.storage.group_planes] in ([(2, 1), (1, 2)], [(1, 2), (2, 1)])
+        got = H.run_trace(eng, steps)
+        H.compare(got, ref, 1e-4, "toy latent %s" % maker.__name__)
+        eng.cache.check_invariants()
+        assert all(eng.cache.free_pages(g) == eng.num_pages for g in range(2))
+    # a fork copies the pages of both groups and the state: the copy goes on as the original would
+    toks = requests["z2"]
+    eng = Engine(model, max_tokens=512, page_size=16, max_requests=4)
+    eng.step([StepEntry("src", toks[:70], [])])
+    eng.fork("src", "dst")
+    eng.step([StepEntry("src", H.random_tokens(83, 9, 1), [])])          # the original moves on with other tokens
+    out = eng.step([StepEntry("dst", toks[70:], list(range(len(toks) - 70)))])
+    err = float((out.cpu().double() - ref["z2"][70:]).abs().max() / ref["z2"].abs().max())
+    assert err < 1e-4, err
