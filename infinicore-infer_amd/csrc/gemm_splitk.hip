@@ -37,7 +37,7 @@ __device__ __forceinline__ uint4 ld16(const uint16_t* p) { return *reinterpret_c
 template <int MT>
 __global__ void __launch_bounds__(kSkThreads)
 gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, float* __restrict__ P,
-                   int M, int N, int K, int lda, int ldw, int chunks_per_slice) {
+                   int M, int N, int K, int lda, int ldw, int chunks_per_slice, int rotate) {
     __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][16 * MT][kSkRowBytes];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
@@ -46,6 +46,18 @@ gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
     const int n_chunks = (K + kSkChunk - 1) / kSkChunk;
     const int c_begin = slice * chunks_per_slice;
     const int c_end = (c_begin + chunks_per_slice < n_chunks) ? c_begin + chunks_per_slice : n_chunks;
+    // Column blocks start their walk over the slice at different chunks and wrap around: blocks that run at the same
+    // time then read different offsets inside the weight rows.  With rows a power of two apart (8 KB, 32 KB) the same
+    // offset in every row falls into few memory channels, and all blocks walking in step queue up there: 4,096 x
+    // 16,384 at 17..64 rows 36.7..38.6 -> 27.6..35.2 us; other shapes (rows of 4,608 bytes and the like) are unchanged.
+    // The order of the sum differs from column block to column block but is fixed for each.
+    const int c_len = c_end - c_begin;
+    const int rot = (rotate && c_len > 0) ? (int)(blockIdx.x % (unsigned)c_len) : 0;
+    auto k_of = [&](int c) {                        // first k of the chunk that is walked as number c
+        int pc = c + rot;
+        if (pc >= c_end) pc -= c_len;
+        return (c < c_end ? pc : c_begin) * kSkChunk;
+    };
 
     // this lane's weight row (clamped: rows beyond N repeat the last one and are not stored)
     const int nrow = (n0 + r < N) ? n0 + r : N - 1;
@@ -79,7 +91,7 @@ gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
     uint4 wreg[4][4], areg[4][MT];
     auto fetch_w = [&](int c, auto set) {
         constexpr int J = decltype(set)::value;
-        const int k0 = c * kSkChunk;
+        const int k0 = k_of(c);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
             const bool ok = c < c_end && k0 + 32 * u + 8 * kq + 8 <= K;
@@ -88,7 +100,7 @@ gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
     };
     auto fetch_a = [&](int c, auto set) {
         constexpr int J = decltype(set)::value;
-        const int k0 = c * kSkChunk;
+        const int k0 = k_of(c);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const bool ok = c < c_end && k0 + a_col[i] + 8 <= K;
@@ -97,7 +109,7 @@ gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
     };
     auto stash = [&](int c, auto set) {            // chunk c, waiting in A register set `set`, into LDS stage set % 2
         constexpr int J = decltype(set)::value;
-        const int k0 = c * kSkChunk;
+        const int k0 = k_of(c);
 #pragma unroll
         for (int i = 0; i < MT; ++i) {
             const uint32_t m = (c < c_end && k0 + a_col[i] + 8 <= K) ? 0xffffffffu : 0u;
@@ -242,6 +254,10 @@ bool splits_ok(const float* P, int S, int M, int N) {
 
 }  // namespace
 
+// For measurements: 0 makes every block walk its slice from the start (1, the default: rotated starts).
+static int g_sk_rotate = 1;
+IC_EXPORT int ic_gemm_splitk_rotate(int on) { g_sk_rotate = on ? 1 : 0; return IC_OK; }
+
 // 1 when the sliced product takes these sizes: 1..64 rows of bfloat16, K a multiple of 8, aligned operands.
 IC_EXPORT int ic_gemm_splitk_supported(int M, int N, int K, int lda, int ldw) {
     return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K;
@@ -283,10 +299,10 @@ IC_EXPORT int ic_gemm_splitk(const void* A, const void* W, float* P, int M, int 
     dim3 grid((N + kSkCols - 1) / kSkCols, n_slices), block(kSkThreads);
     const uint16_t* a = (const uint16_t*)A;
     const uint16_t* w = (const uint16_t*)W;
-    if (M <= 16) hipLaunchKernelGGL(gemm_splitk_kernel<1>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per);
-    else if (M <= 32) hipLaunchKernelGGL(gemm_splitk_kernel<2>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per);
-    else if (M <= 48) hipLaunchKernelGGL(gemm_splitk_kernel<3>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per);
-    else hipLaunchKernelGGL(gemm_splitk_kernel<4>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per);
+    if (M <= 16) hipLaunchKernelGGL(gemm_splitk_kernel<1>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
+    else if (M <= 32) hipLaunchKernelGGL(gemm_splitk_kernel<2>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
+    else if (M <= 48) hipLaunchKernelGGL(gemm_splitk_kernel<3>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
+    else hipLaunchKernelGGL(gemm_splitk_kernel<4>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
     return ic_launch_status();
 }
 

@@ -127,7 +127,7 @@ def swiglu(gate_up, out):
 
 def copy_pages(planes, src, dst):
     """planes[..., dst[i], :, :, :] = planes[..., src[i], :, :, :] for a cache group's planes
-    [slots, 2, pages, kv_heads, page_size, head_dim] (contiguous); src, dst: int32 page ids on the device."""
+    [slots, planes, pages, kv_heads, page_size, head_dim] (contiguous); src, dst: int32 page ids on the device."""
     _dev(planes, src, dst)
     _i32(src, "src")
     _i32(dst, "dst")
