@@ -22,8 +22,22 @@
 // O^T = V^T P^T slot (h, e) of 16-key chunk c stands for key 16c + 4h + e
 // (e < 4) and 16c + 8 + 4h + (e - 4) (e >= 4), which is where D left P^T.
 //
+// A query tile's walk over the keys may also be cut into parts that run as blocks of their own (GROUPS == 1): the
+// grid then holds `parts` blocks per (tile, head), block `part` walks its share of the tile's key tiles (at least
+// part_len of them a part; blocks beyond a tile's number of parts leave at once), writes its running maximum, sum
+// and O^T to scratch memory and counts itself in; the block that arrives last merges the others' results into its
+// own and writes the output.  Nobody waits for anybody.  With few blocks the longest tile's walk is the kernel's
+// time (a 2,048-token prompt: 32 key tiles one after the other while most of the chip has run dry), and parts cut it
+// without the 8-wave blocks of GROUPS == 2.
+//
 // Cache layout of one layer: K and V planes [num_pages, n_kv_heads, page_size, head_dim].
 #include "common.h"
+
+// Arrival counters of the split walk, one per (tile, head): zero when the library is loaded, and put back to zero
+// by the block that merges.  Launches that split and overlap in time on one device would share them: the engine
+// issues a step's kernels on one stream.
+constexpr int kPfCounters = 1 << 16;
+__device__ int g_pf_arrivals[kPfCounters];
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -47,7 +61,8 @@ __global__ void __launch_bounds__(256 * GROUPS, (GROUPS == 1 && DH <= 64) ? 3 : 
 attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t* __restrict__ out, int out_stride,
                          const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                          const int* __restrict__ block_tables, int bt_stride, const int4* __restrict__ tiles,
-                         int n_tiles, int nh, int nkvh, int page_shift, float scale_log2e, int window) {
+                         int n_tiles, int nh, int nkvh, int page_shift, float scale_log2e, int window,
+                         int parts, int part_len, float* __restrict__ scratch) {
     constexpr int NC = DH / 16;           // 16-wide chunks of the head dimension
     constexpr int ND = DH / 32;           // 32-row tiles of O^T
     constexpr int KS = DH + kPfPad;       // row stride of Ks (elements): 16-byte reads of 8 consecutive rows cover all banks
@@ -70,8 +85,10 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     // blocks are dealt to the 8 XCDs in turn (block b runs on XCD b % 8) every XCD gets an equal share of
     // every length.  A head's tiles then meet on few XCDs (two of them with 36 heads), so its keys still
     // stay in those L2s.
-    const int h = blockIdx.x % nh;
-    const int4 tile = tiles[blockIdx.x / nh];
+    const int part = (GROUPS == 1 && parts > 1) ? (int)(blockIdx.x / ((unsigned)nh * (unsigned)n_tiles)) : 0;
+    const int slot = (int)blockIdx.x - part * nh * n_tiles;          // (tile, head)
+    const int h = slot % nh;
+    const int4 tile = tiles[slot / nh];
     const int req = tile.x, row0 = tile.y, n_rows = tile.z, pos0 = tile.w;
     const int kvh = h / (nh / nkvh);
     const int* bt = block_tables + (size_t)req * bt_stride;
@@ -90,8 +107,21 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     int first_key = 0;
     if (window > 0 && pos0 - window + 1 > 0) first_key = pos0 - window + 1;
 
+    // this block's share of the tile's key tiles
+    const int kt0 = (first_key / kPfKeys) * kPfKeys;
+    const int n_kt = (last_key - kt0) / kPfKeys + 1;
+    int n_parts = 1;
+    if (GROUPS == 1 && parts > 1) {
+        n_parts = (n_kt + part_len - 1) / part_len;
+        n_parts = n_parts < parts ? n_parts : parts;
+        if (part >= n_parts) return;                         // (the whole block: nobody is left at a barrier)
+    }
+    const int kb_begin = kt0 + kPfKeys * (int)((long long)n_kt * part / n_parts);
+    const int kb_end = kt0 + kPfKeys * (int)((long long)n_kt * (part + 1) / n_parts);      // one past this part's last tile
+
     // page ids of the keys this block reads, staged once (one memory hop less per tile)
-    const int page_lo = first_key >> page_shift, page_hi = last_key >> page_shift;
+    const int page_lo = (kb_begin > first_key ? kb_begin : first_key) >> page_shift;
+    const int page_hi = (kb_end - 1 < last_key ? kb_end - 1 : last_key) >> page_shift;
     // STAGED is chosen by the host from the block table's width: a run-time choice between the
     // two arrays would turn every lookup into a flat load, and waiting for a flat load also
     // waits for the key and value loads in flight.
@@ -192,13 +222,12 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
 
     const uint16_t* const Ks = Ks_all + grp * KT;
     const uint16_t* const Vs = Vs_all + grp * VT;
-    const int kt0 = (first_key / kPfKeys) * kPfKeys;
-    fetch(kt0);
-    for (int kb = kt0; kb <= last_key; kb += STEP) {
+    fetch(kb_begin);
+    for (int kb = kb_begin; kb < kb_end; kb += STEP) {
         __syncthreads();                                     // the previous step's readers are done
         stash();
         __syncthreads();
-        if (kb + STEP <= last_key) fetch(kb + STEP);         // in flight while this step is used
+        if (kb + STEP < kb_end) fetch(kb + STEP);            // in flight while this step is used
         const int kt = kb + kPfKeys * grp;                   // this group's key tile
         if (!wave_ok || kt > wave_last) continue;            // nothing this wave may see
         if (window > 0 && kt + kPfKeys - 1 < wave_first - window + 1) continue;
@@ -309,6 +338,47 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             for (int r = 0; r < 16; ++r) oacc[i][r] = oacc[i][r] * c0 + mbuf[2 + 16 * i + r] * c1;
     }
     }
+    // ---- a walk cut into parts: hand the state over, and the block that arrives last merges and writes ----------
+    if (GROUPS == 1 && n_parts > 1) {
+        __shared__ int arrived;
+        constexpr int PF = kPfWaveThreads * MERGE_F;          // floats of one part: [field][thread], so that stores coalesce
+        // The parts of a tile run on different XCDs, whose L2 caches do not see each other's lines: the state goes out
+        // with device-scope stores (written through) and comes in with device-scope loads (not served from this XCD's
+        // L2), so that no cache has to be written back or invalidated as a whole, which a device-scope fence would do
+        // (with fences the kernel took three times as long).  The count is a device-scope atomic.
+        float* const mine = scratch + ((size_t)slot * parts + part) * PF;
+        auto put = [](float* p, float v) { __hip_atomic_store(p, v, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+        auto get = [](const float* p) { return __hip_atomic_load(p, __ATOMIC_RELAXED, __HIP_MEMORY_SCOPE_AGENT); };
+        put(mine + tid, m);
+        put(mine + kPfWaveThreads + tid, l);
+#pragma unroll
+        for (int i = 0; i < ND; ++i)
+#pragma unroll
+            for (int r = 0; r < 16; ++r) put(mine + (2 + 16 * i + r) * kPfWaveThreads + tid, oacc[i][r]);
+        // a thread's stores must have completed before the block counts itself in: the barrier alone does not wait
+        // for stores to memory (waves of a block share their unit's cache, so a barrier need not)
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
+        __syncthreads();
+        if (tid == 0) arrived = atomicAdd(&g_pf_arrivals[slot], 1);
+        __syncthreads();
+        if (arrived != n_parts - 1) return;
+        if (tid == 0) g_pf_arrivals[slot] = 0;               // for the next launch
+        for (int p = 0; p < n_parts; ++p) {
+            if (p == part) continue;
+            const float* other = scratch + ((size_t)slot * parts + p) * PF;
+            const float m1 = get(other + tid), l1 = get(other + kPfWaveThreads + tid);
+            const float m_new = fmaxf(m, m1);
+            const float mc = ((m_new == -INFINITY) ? 0.f : m_new) * scale_log2e;
+            const float c0 = __builtin_amdgcn_exp2f(m * scale_log2e - mc), c1 = __builtin_amdgcn_exp2f(m1 * scale_log2e - mc);
+            l = l * c0 + l1 * c1;
+            m = m_new;
+#pragma unroll
+            for (int i = 0; i < ND; ++i)
+#pragma unroll
+                for (int r = 0; r < 16; ++r)
+                    oacc[i][r] = oacc[i][r] * c0 + get(other + (2 + 16 * i + r) * kPfWaveThreads + tid) * c1;
+        }
+    }
     if (!row_ok) return;
     const float inv = 1.0f / l;
     uint16_t* op = out + (size_t)(row0 + my_row) * out_stride + (size_t)h * DH;
@@ -330,12 +400,49 @@ IC_EXPORT int ic_attn_prefill_supported(int dtype, int dh, int page_size) {
 
 IC_EXPORT int ic_attn_prefill_tile_rows() { return kPfRows; }
 
+// Floats of scratch memory that a walk cut into `parts` needs: every (tile, head, part) keeps a maximum, a sum and O^T per row.
+IC_EXPORT long long ic_attn_prefill_scratch_floats(int n_tiles, int nh, int dh, int parts) {
+    if (n_tiles <= 0 || nh <= 0 || parts <= 1 || (dh != 64 && dh != 128)) return 0;
+    return (long long)n_tiles * nh * parts * kPfWaveThreads * (2 + dh / 2);
+}
+
+// How to cut the walks of a step whose longest query tile sees `max_keys` keys: parts per tile (1: no cut) and key tiles
+// per part.  From a sweep over 16..48 heads of 64 and 32..40 of 128, prompts of 300..4,096 tokens and portions of 256..1,024
+// after 1,024..3,584 tokens, against one and two wave groups:
+//  * parts pay when walks are long (24 key tiles and more) and blocks are few: as many parts as keep about 4.5 blocks a compute
+//    unit at head size 64 and 2 at head size 128 (what stays resident there), at most 4, each of 6 key tiles or more;
+//  * portions after a long past gain most (16 heads, 512 tokens after 3,584: 54 -> 26 us; 36 heads: 54 -> 41; 32:2 x 128: 83 -> 52),
+//    whole prompts little (36 heads, 2,048 tokens: 43 -> 41 us) or nothing;
+//  * two parts do no better than two wave groups where those run (up to 2 blocks a unit), so they keep that case.
+IC_EXPORT int ic_attn_prefill_parts(int n_tiles, int nh, int dh, int max_keys, int compute_units, int* part_len) {
+    const int longest = (max_keys + kPfKeys - 1) / kPfKeys;
+    const long long blocks = (long long)n_tiles * nh;
+    int len = longest > 0 ? longest : 1, parts = 1;
+    if (compute_units > 0 && blocks > 0 && blocks <= kPfCounters && longest >= 24 && (dh == 64 || dh == 128)) {
+        const long long room = dh == 64 ? 9LL * compute_units / 2 : 2LL * compute_units;
+        long long p = room / blocks;
+        p = p > 4 ? 4 : p;
+        p = p > longest / 6 ? longest / 6 : p;
+        if (p == 2 && blocks <= 2LL * compute_units) p = 1;
+        if (p >= 2) {
+            parts = (int)p;
+            len = (longest + parts - 1) / parts;
+            len = len < 6 ? 6 : len;
+        }
+    }
+    if (part_len) *part_len = len;
+    return parts;
+}
+
 // tiles: int32 [n_tiles, 4] = (request row of block_tables, first token row, rows <= 128, position of the first row).
-// groups: 1 or 2 wave groups per query tile, 0 = chosen from the number of blocks.
-IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int out_stride, int dtype,
-                                     const void* kcache, const void* vcache, const int* block_tables,
-                                     int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
-                                     int page_size, float scale, int window, int groups, hipStream_t stream) {
+// groups: 1 or 2 wave groups per query tile, 0 = chosen from the number of blocks.  parts > 1 (one group only): the grid
+// holds `parts` blocks per (tile, head) and a tile's walk is cut into up to that many parts of at least part_len key
+// tiles; scratch then holds ic_attn_prefill_scratch_floats(...) floats.
+IC_EXPORT int ic_attn_prefill_split(const void* q, int q_stride, void* out, int out_stride, int dtype,
+                                    const void* kcache, const void* vcache, const int* block_tables,
+                                    int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
+                                    int page_size, float scale, int window, int groups, int parts, int part_len,
+                                    float* scratch, long long scratch_floats, hipStream_t stream) {
     if (n_tiles <= 0) return IC_OK;
     if (!ic_attn_prefill_supported(dtype, dh, page_size)) return IC_ERR_UNSUPPORTED;
     int page_shift = 0;
@@ -343,6 +450,13 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || nh > 65535 || groups < 0 || groups > 2) return IC_ERR_ARG;
     if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7) ||
         ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15) || ((uintptr_t)tiles & 15)) return IC_ERR_ARG;
+    if (parts < 1) parts = 1;
+    if (parts > 1) {
+        if (groups == 2 || part_len < 1 || parts > 64 || (long long)nh * n_tiles > kPfCounters || !scratch ||
+            ((uintptr_t)scratch & 15) || scratch_floats < ic_attn_prefill_scratch_floats(n_tiles, nh, dh, parts) ||
+            (long long)nh * n_tiles * parts > 0x7fffffffLL) return IC_ERR_ARG;
+        groups = 1;
+    }
     const float sl2 = scale * 1.4426950408889634f;
     const bool staged = bt_stride <= kPfMaxPages;       // a block never needs more page ids than a request has
     // Few blocks (up to 2 per compute unit; measured with 16..64 heads of 64 and 32..40 of 128 over 512..4,096
@@ -356,12 +470,13 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
         else cus = 256;
     }
     const bool two_groups = groups ? groups == 2 : (long long)nh * n_tiles <= 2LL * cus;
-    dim3 grid((unsigned)nh * (unsigned)n_tiles);
+    dim3 grid((unsigned)nh * (unsigned)n_tiles * (unsigned)parts);
     const bool page64 = page_size >= kPfKeys;            // (a power of two) a 64-key tile lies in one page
 #define IC_PF_LAUNCH(DD, ST, GG, PP)                                                                                   \
     hipLaunchKernelGGL((attn_prefill_mfma_kernel<DD, ST, GG, PP>), grid, dim3(256 * GG), 0, stream, (const uint16_t*)q, \
                        q_stride, (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
-                       block_tables, bt_stride, (const int4*)tiles, n_tiles, nh, nkvh, page_shift, sl2, window)
+                       block_tables, bt_stride, (const int4*)tiles, n_tiles, nh, nkvh, page_shift, sl2, window,      \
+                       parts, part_len, scratch)
 #define IC_PF_GROUPS(DD, ST) do { if (two_groups) { if (page64) IC_PF_LAUNCH(DD, ST, 2, true); else IC_PF_LAUNCH(DD, ST, 2, false); } \
                                   else { if (page64) IC_PF_LAUNCH(DD, ST, 1, true); else IC_PF_LAUNCH(DD, ST, 1, false); } } while (0)
     if (dh == 64) { if (staged) IC_PF_GROUPS(64, true); else IC_PF_GROUPS(64, false); }
@@ -371,6 +486,14 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
     else
         return IC_ERR_UNSUPPORTED;
     return ic_launch_status();
+}
+
+IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int out_stride, int dtype,
+                                     const void* kcache, const void* vcache, const int* block_tables,
+                                     int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
+                                     int page_size, float scale, int window, int groups, hipStream_t stream) {
+    return ic_attn_prefill_split(q, q_stride, out, out_stride, dtype, kcache, vcache, block_tables, bt_stride, tiles,
+                                 n_tiles, nh, nkvh, dh, page_size, scale, window, groups, 1, 0, nullptr, 0, stream);
 }
 
 IC_EXPORT int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype,

@@ -29,7 +29,7 @@ inline int dtype_size(int dtype) { return dtype == IC_BF16 ? 2 : 4; }
 struct Workspace {
     // byte offsets into the caller's workspace
     size_t residual, normed, qkv, attn_out, mixer_out, ffn_out, mixer_tail, mixer_sumsq, ffn_tail, ffn_sumsq, gate_up, act,
-        part_acc, part_ml, head_in, tail_parts, total;
+        part_acc, part_ml, head_in, tail_parts, tile_parts, total;
 };
 
 // Rows whose norm is half done: values = x * w, sums of squares per column block; the row factor
@@ -73,6 +73,13 @@ struct IcDecoder {
         return split_answer;
     }
 
+    // into how many parts the walks of a step's prompt tiles are cut (1: not at all), and key tiles per part
+    int tile_parts_for(const IcStepBatch& b, const IcAttention& a, int* part_len) const {
+        int keys = b.max_position + 1;
+        if (a.window > 0 && a.window + ic_attn_prefill_tile_rows() < keys) keys = a.window + ic_attn_prefill_tile_rows();
+        return ic_attn_prefill_parts(b.n_prefill_tiles, a.n_heads, a.head_dim, keys, meta.compute_units, part_len);
+    }
+
     Workspace layout(const IcStepBatch& b) const {
         const size_t T = (size_t)b.n_tokens, d = (size_t)meta.hidden, ds = (size_t)dtype_size(meta.dtype);
         const int parts = ic_gemm_nt_residual_parts(meta.hidden);
@@ -109,6 +116,14 @@ struct IcDecoder {
                 slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, l.ffn.intermediate));
             }
         w.tail_parts = take(slices * T * d * 4);
+        size_t cut = 0;              // the states of prompt tiles whose walk over the keys is cut into parts
+        if (meta.dtype == IC_BF16 && b.n_prefill_tiles > 0)
+            for (const IcLayer& l : layers) {
+                int len = 0;
+                const int p = tile_parts_for(b, l.attention, &len);
+                cut = std::max(cut, (size_t)ic_attn_prefill_scratch_floats(b.n_prefill_tiles, l.attention.n_heads, l.attention.head_dim, p));
+            }
+        w.tile_parts = take(cut * 4);
         w.total = o;
         return w;
     }
@@ -242,8 +257,12 @@ struct IcDecoder {
                     if (st) return fail(st, "attention of single tokens", i);
                 }
                 if (use_pre) {
-                    st = ic_attn_prefill_groups(qkv, width, attn_out, ow, dt, e.k_cache, e.v_cache, tables, bts, b.prefill_tiles,
-                                                n_tiles, A.n_heads, A.n_kv_heads, A.head_dim, ps, A.softmax_scale, A.window, 0, stream);
+                    int part_len = 0;
+                    const int parts = tile_parts_for(b, A, &part_len);
+                    st = ic_attn_prefill_split(qkv, width, attn_out, ow, dt, e.k_cache, e.v_cache, tables, bts, b.prefill_tiles,
+                                               n_tiles, A.n_heads, A.n_kv_heads, A.head_dim, ps, A.softmax_scale, A.window, 0, parts,
+                                               part_len, (float*)(base + ws.tile_parts),
+                                               ic_attn_prefill_scratch_floats(n_tiles, A.n_heads, A.head_dim, parts), stream);
                     if (st) return fail(st, "attention of prompt portions", i);
                 }
             }

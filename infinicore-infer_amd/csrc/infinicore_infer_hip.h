@@ -49,6 +49,14 @@ int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int 
 // The same with the number of wave groups per query tile given: 2 halves the longest tile's walk over the keys (few blocks), 1 keeps more blocks resident (many blocks), 0 chooses.
 int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, hipStream_t stream);
 
+// The same with a query tile's walk over the keys cut into parts that run as blocks of their own (one wave group): the grid holds
+// `parts` blocks per (tile, head), a part walks at least part_len key tiles of 64, the block that arrives last merges the parts
+// through `scratch` (ic_attn_prefill_scratch_floats floats).  ic_attn_prefill_parts proposes parts and part_len for a step whose
+// longest tile sees max_keys keys (1: no cut).  Launches that cut and overlap in time on one device share the arrival counters: use one stream.
+long long ic_attn_prefill_scratch_floats(int n_tiles, int nh, int dh, int parts);
+int ic_attn_prefill_parts(int n_tiles, int nh, int dh, int max_keys, int compute_units, int* part_len);
+int ic_attn_prefill_split(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, int parts, int part_len, float* scratch, long long scratch_floats, hipStream_t stream);
+
 // ---- gemm.hip ---------------------------------------------------------------------------------------
 // A norm y = x * rsqrt(mean(x^2) + eps) * w between two products of M <= 16 rows can be split over them: the
 // product before it adds its result to the residual stream, stores x * w and the sums of x^2 per row and

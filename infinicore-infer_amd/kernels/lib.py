@@ -102,6 +102,9 @@ _SIGNATURES = {
     "ic_attn_prefill_tile_rows": [],
     "ic_attn_prefill": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _P],
     "ic_attn_prefill_groups": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
+    "ic_attn_prefill_scratch_floats": [_I, _I, _I, _I],
+    "ic_attn_prefill_parts": [_I, _I, _I, _I, _I, _c.POINTER(_I)],
+    "ic_attn_prefill_split": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _LL, _P],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_argmax_static_max_rows": [],
@@ -138,7 +141,7 @@ _SIGNATURES = {
 }
 _RESTYPES = {"ic_decoder_create": _P, "ic_decoder_create_error": _c.c_char_p, "ic_decoder_destroy": None,
              "ic_decoder_last_error": _c.c_char_p, "ic_decoder_workspace_bytes": _LL, "ic_decoder_step_ints": _LL,
-             "ic_peak_mfma_bf16": _LL}
+             "ic_peak_mfma_bf16": _LL, "ic_attn_prefill_scratch_floats": _LL}
 
 
 def get_lib():

@@ -247,19 +247,41 @@ def attention_prefill_tile_rows() -> int:
     return get_lib().ic_attn_prefill_tile_rows()
 
 
+def attention_prefill_parts(n_tiles: int, n_heads: int, head_dim: int, max_keys: int, compute_units: int):
+    """(parts, part_len): into how many blocks of their own to cut the query tiles' walks over the keys when the longest
+    tile of the step sees ``max_keys`` keys (1: no cut), and how many key tiles of 64 a part holds at least."""
+    import ctypes
+    part_len = ctypes.c_int(0)
+    parts = get_lib().ic_attn_prefill_parts(int(n_tiles), int(n_heads), int(head_dim), int(max_keys), int(compute_units),
+                                            ctypes.byref(part_len))
+    return int(parts), int(part_len.value)
+
+
+def attention_prefill_scratch_floats(n_tiles: int, n_heads: int, head_dim: int, parts: int) -> int:
+    return int(get_lib().ic_attn_prefill_scratch_floats(int(n_tiles), int(n_heads), int(head_dim), int(parts)))
+
+
 def attention_prefill(q, out, kcache, vcache, block_tables, tiles, n_tiles, n_heads, n_kv_heads, head_dim,
-                      page_size, scale: float, window: int = 0, groups: int = 0):
+                      page_size, scale: float, window: int = 0, groups: int = 0, parts: int = 1, part_len: int = 0,
+                      scratch=None):
     """Matrix-core attention of prompt portions.  tiles: int32 [n, 4] rows of
     (request row in block_tables, first token row, rows <= tile_rows, first position).
-    groups: wave groups per query tile (1 or 2); 0 lets the kernel choose from the number of blocks."""
+    groups: wave groups per query tile (1 or 2); 0 lets the kernel choose from the number of blocks.
+    parts > 1: every tile's walk over the keys is cut into up to ``parts`` blocks of at least ``part_len`` key tiles
+    that meet through ``scratch`` (float32, attention_prefill_scratch_floats(...) elements)."""
     _need(groups in (0, 1, 2), "attention_prefill: groups must be 0, 1 or 2")
     _attn_common(q, out, kcache, vcache, block_tables, n_heads, n_kv_heads, head_dim, page_size)
     _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.dim() == 2 and tiles.shape[1] == 4
           and tiles.shape[0] >= n_tiles, "attention_prefill: tiles must be int32 [n, 4]")
-    check(get_lib().ic_attn_prefill_groups(
+    if parts > 1:
+        _dev(scratch)
+        _need(scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous(),
+              "attention_prefill: a cut walk needs float32 scratch memory")
+    check(get_lib().ic_attn_prefill_split(
         q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype), kcache.data_ptr(),
         vcache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), tiles.data_ptr(), n_tiles,
-        n_heads, n_kv_heads, head_dim, page_size, float(scale), int(window or 0), int(groups), _stream()),
+        n_heads, n_kv_heads, head_dim, page_size, float(scale), int(window or 0), int(groups), int(parts), int(part_len),
+        scratch.data_ptr() if parts > 1 else None, scratch.numel() if parts > 1 else 0, _stream()),
         "attention_prefill")
 
 

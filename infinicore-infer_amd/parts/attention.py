@@ -146,5 +146,14 @@ class Attention(Mixer):
                                  ctx.token_req, ctx.positions, part_acc, part_ml, *args, self.scale,
                                  self.window, n_split)
         if use_pre:
+            # few blocks and long walks over the keys: the tiles' walks are cut into parts (the library's rule)
+            keys = ctx.max_position + 1
+            if self.window:
+                keys = min(keys, self.window + ops.attention_prefill_tile_rows())
+            parts, part_len = ops.attention_prefill_parts(n_tiles, self.nh, self.dh, keys, ctx.cu_count)
+            scratch = None
+            if parts > 1:
+                scratch = ctx.ws.buffer("attn_tile_parts", (ops.attention_prefill_scratch_floats(n_tiles, self.nh, self.dh, parts),),
+                                        torch.float32)
             ops.attention_prefill(q, out, cache.k, cache.v, cache.block_tables, ctx.prefill_tiles, n_tiles,
-                                  *args, self.scale, self.window)
+                                  *args, self.scale, self.window, parts=parts, part_len=part_len, scratch=scratch)

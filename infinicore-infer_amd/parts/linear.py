@@ -59,6 +59,9 @@ def linear(x, w, out, impl: str = "auto", alpha: float = 1.0):
         x = x.materialize()
     if w.dtype != x.dtype:
         # a matrix stored in 32-bit stays so: compute this product in float32
+        # (w is the 32-bit one, so only the few activations are converted; no copy of the matrix is made)
+        if out.dtype == torch.float32:
+            return _library(x.to(torch.float32), w.to(torch.float32), out, alpha)
         tmp = torch.empty(out.shape, dtype=torch.float32, device=out.device)
         _library(x.to(torch.float32), w.to(torch.float32), tmp, alpha)
         out.copy_(tmp)

@@ -417,3 +417,54 @@ def test_recorded_steps_hold_a_bounded_amount_of_memory(tmp_path_factory, native
             ref.step([StepEntry(r, [1 + i], [0]) for i, r in enumerate(ids[:2])])
     want = ref.step([StepEntry(r, [9], [0]) for r in ids[:2]])      # other batches, other kernels: equal to rounding
     assert float((again - want).abs().max()) <= H.BF16_TOL * float(want.abs().max())
+
+
+@pytest.mark.parametrize("native", [True, False])
+def test_prompt_portions_after_a_long_past_walk_their_keys_in_parts(tmp_path_factory, native):
+    """A prompt of 2,000 tokens in portions of 512 beside a second request: from the fourth portion on the query
+    tiles see 24 and more key tiles and there are few blocks, so each tile's walk over the keys is cut into parts
+    that blocks of their own take (head size 64, grouped queries, page size 64, bfloat16).  Compared with the plain
+    implementation at the first, the last and some other places of every portion."""
+    import os
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.kernels import ops
+    from infinicore_infer_amd.weights import write_random_model
+    from plain_model import plain_forward, round_bf16
+    cfg = dict(model_type="minicpm", vocab_size=1009, hidden_size=256, num_hidden_layers=2, num_attention_heads=4,
+               num_key_value_heads=2, intermediate_size=384, max_position_embeddings=2048, rms_norm_eps=1e-5,
+               rope_theta=10000.0, scale_emb=4, dim_model_base=64, scale_depth=1.2, tie_word_embeddings=False, eos_token_id=2)
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "model_long_past")
+    if not os.path.exists(os.path.join(folder, "config.json")):
+        write_random_model(folder, cfg, seed=21, std=0.05)
+    sd = H.load_state_dict(folder)
+    a, b = H.random_tokens(1009, 2000, 5), H.random_tokens(1009, 700, 6)
+    cuts_a = [0, 512, 1024, 1536, 1900, 2000]
+    cuts_b = [0, 0, 300, 300, 700, 700]                    # b's portions ride along in the third and fifth step
+    steps, want_a, want_b = [], [], []
+    for i in range(5):
+        ents = []
+        n = cuts_a[i + 1] - cuts_a[i]
+        w = sorted({0, 1, n // 2, n - 2, n - 1})
+        ents.append({"id": "a", "tokens": a[cuts_a[i]:cuts_a[i + 1]], "want": w})
+        want_a += [cuts_a[i] + j for j in w]
+        nb = cuts_b[i + 1] - cuts_b[i]
+        if nb:
+            wb = [0, nb - 1]
+            ents.append({"id": "b", "tokens": b[cuts_b[i]:cuts_b[i + 1]], "want": wb})
+            want_b += [cuts_b[i] + j for j in wb]
+        steps.append({"step": i, "entries": ents, "end": []})
+    steps[-1]["end"] = ["a", "b"]
+    engine = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=2048 + 704, page_size=64, max_requests=2, use_native=native)
+    assert (engine.native is not None) == native
+    # the rule really cuts these steps: 4 and 3 tiles of the first request (and 4 of the second) with 4 heads
+    assert ops.attention_prefill_parts(4, 4, 64, 2048, engine.cu_count)[0] == 4
+    assert ops.attention_prefill_parts(3 + 4, 4, 64, 1900, engine.cu_count)[0] == 4
+    got = H.run_trace(engine, steps)
+    ref_a = plain_forward(cfg, sd, a, rnd=round_bf16, rows=want_a)
+    ref_b = plain_forward(cfg, sd, b, rnd=round_bf16, rows=want_b)
+    ref = {"a": {p: ref_a[i] for i, p in enumerate(want_a)}, "b": {p: ref_b[i] for i, p in enumerate(want_b)}}
+    assert sorted(got) == sorted([("a", p) for p in want_a] + [("b", p) for p in want_b])
+    scale = float(max(ref_a.abs().max(), ref_b.abs().max()))
+    for (rid, pos), row in sorted(got.items()):
+        err = float((row.double() - ref[rid][pos]).abs().max()) / scale
+        assert err <= H.BF16_TOL, "request %s position %d differs by %.3g of the largest logit" % (rid, pos, err)

@@ -156,9 +156,11 @@ def test_rope_kv_write(dtype, nh, nkvh, dh, rot, page):
         _close(got[:, :nh][..., perm], adj, dtype)
 
 
-def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_width=0, groups=0, n_split=3):
+def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_width=0, groups=0, n_split=3, parts=None):
     """lens: list of (past, new) per request.  Returns (got, want) [T, nh*dh].  table_width pads
-    the block tables with unused columns; groups is passed to the prompt-portion kernel."""
+    the block tables with unused columns; groups is passed to the prompt-portion kernel; parts = (parts, part_len)
+    cuts the prompt tiles' walks over the keys (the kernel is then launched twice: its arrival counters must come
+    back to zero)."""
     ops = _ops()
     g = torch.Generator().manual_seed(seed)
     scale = 1.0 / math.sqrt(dh)
@@ -204,7 +206,14 @@ def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_w
                 tiles += [r, row0 + o, min(rows, new - o), past + o]
             row0 += new
         tl = torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 4)
-        ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0, groups)
+        if parts:
+            scratch = torch.full((ops.attention_prefill_scratch_floats(tl.shape[0], nh, dh, parts[0]),), float("nan"), device=DEV)
+            for _ in range(2):
+                out.zero_()
+                ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0, 1,
+                                      parts=parts[0], part_len=parts[1], scratch=scratch)
+        else:
+            ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0, groups)
     return out, torch.cat(want)
 
 
@@ -237,6 +246,37 @@ def test_attention_prefill_mfma(nh, nkvh, dh, page, window, groups):
     lens = [(0, 2), (0, 129), (130, 64), (64, 33), (15, 2), (257, 300), (5, 128)]
     got, want = _attention_case(torch.bfloat16, nh, nkvh, dh, page, lens, window, 13, "prefill", groups=groups)
     _close(got, want, torch.bfloat16, factor=3)
+
+
+@pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (3, 1, 64, 32), (4, 2, 128, 16), (4, 4, 128, 64)])
+@pytest.mark.parametrize("window", [None, 300])
+@pytest.mark.parametrize("parts", [(2, 1), (3, 2), (4, 1), (8, 3)])
+def test_attention_prefill_with_the_walk_over_the_keys_cut_into_parts(nh, nkvh, dh, page, window, parts):
+    """Blocks of their own walk parts of a query tile's keys and the last one to arrive merges them: tiles with fewer
+    key tiles than parts, tiles that start inside a page, a request of two tokens, two launches in a row."""
+    lens = [(0, 2), (0, 129), (130, 64), (700, 140), (257, 300), (5, 128), (1000, 33)]
+    got, want = _attention_case(torch.bfloat16, nh, nkvh, dh, page, lens, window, 23, "prefill", parts=parts)
+    _close(got, want, torch.bfloat16, factor=3)
+
+
+def test_attention_prefill_parts_rule_and_its_refusals():
+    ops = _ops()
+    assert ops.attention_prefill_parts(16, 36, 64, 2048, 256) == (2, 16)         # the benchmark's prompt: 576 blocks of 32 key tiles
+    assert ops.attention_prefill_parts(4, 36, 64, 2048, 256)[0] == 4             # a portion of 512 after 1,536
+    assert ops.attention_prefill_parts(4, 36, 64, 1024, 256)[0] == 1             # short walks are left whole
+    assert ops.attention_prefill_parts(32, 36, 64, 4096, 256)[0] == 1            # many blocks too
+    assert ops.attention_prefill_parts(16, 32, 128, 2048, 256)[0] == 1 and ops.attention_prefill_parts(4, 40, 128, 4096, 256)[0] == 3
+    assert ops.attention_prefill_scratch_floats(4, 36, 64, 4) == 4 * 36 * 4 * 256 * 34
+    q = torch.zeros(128, 64, dtype=torch.bfloat16, device=DEV)
+    kc = torch.zeros(2, 1, 64, 64, dtype=torch.bfloat16, device=DEV)
+    bt = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
+    tl = torch.tensor([[0, 0, 128, 0]], dtype=torch.int32, device=DEV)
+    small = torch.zeros(16, device=DEV)
+    with pytest.raises(ops.KernelError):        # scratch memory too small for two parts
+        ops.attention_prefill(q, torch.zeros_like(q), kc, kc, bt, tl, 1, 1, 1, 64, 64, 0.125, 0, 1, parts=2, part_len=1, scratch=small)
+    with pytest.raises(ops.KernelError):        # parts go with one wave group only
+        ops.attention_prefill(q, torch.zeros_like(q), kc, kc, bt, tl, 1, 1, 1, 64, 64, 0.125, 0, 2, parts=2, part_len=1,
+                              scratch=torch.zeros(2 * 256 * 34, device=DEV))
 
 
 @pytest.mark.parametrize("impl,dtype,nh,nkvh,dh", [("decode", torch.bfloat16, 6, 6, 64), ("decode", torch.float32, 4, 4, 128),
