@@ -20,7 +20,7 @@ constexpr int kDecMaxPages = 1024;   // page ids of one block's keys staged in L
 template <typename T> struct Vec16;
 template <> struct Vec16<float> {
     static constexpr int N = 4;
-    __device__ static uint4 raw(const float* p) { return *reinterpret_cast<const uint4*>(p); }
+    __device__ static uint4 raw(const float* p) { return load_stream16(p); }
     __device__ static void unpack(const uint4& v, float* o) {
         o[0] = __uint_as_float(v.x); o[1] = __uint_as_float(v.y);
         o[2] = __uint_as_float(v.z); o[3] = __uint_as_float(v.w);
@@ -29,7 +29,7 @@ template <> struct Vec16<float> {
 };
 template <> struct Vec16<bf16> {
     static constexpr int N = 8;
-    __device__ static uint4 raw(const bf16* p) { return *reinterpret_cast<const uint4*>(p); }
+    __device__ static uint4 raw(const bf16* p) { return load_stream16(p); }
     __device__ static void unpack(const uint4& v, float* o) {
         o[0] = __uint_as_float(v.x << 16); o[1] = __uint_as_float(v.x & 0xffff0000u);
         o[2] = __uint_as_float(v.y << 16); o[3] = __uint_as_float(v.y & 0xffff0000u);
@@ -402,6 +402,9 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
                 const size_t off = ok ? row_of(key) + 8 * lg : 0;
 #pragma unroll
                 for (int c = 0; c < NC; ++c) {
+                    // (plain loads: a wave's load covers 64 bytes of each of 16 key rows, half a cache line, and the other
+                    // half comes with the next load; without the caches keeping the line it would be fetched twice.
+                    // The values below and both planes in the kernel above are read in whole rows and are streamed.)
                     if (ok) kreg[s2][c].u = *reinterpret_cast<const uint4*>(kbase + off + 32 * c);
                     else kreg[s2][c].u = make_uint4(0, 0, 0, 0);
                 }
@@ -412,7 +415,7 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
                 const int vkey = idx / (DH / 8), oct = idx - vkey * (DH / 8);
                 const int key = kt + vkey;
                 vreg[i] = make_uint4(0, 0, 0, 0);
-                if (tile < n_tiles && key < hi) vreg[i] = *reinterpret_cast<const uint4*>(vbase + row_of(key) + oct * 8);
+                if (tile < n_tiles && key < hi) vreg[i] = load_stream16(vbase + row_of(key) + oct * 8);
             }
         };
         auto stash = [&]() {
