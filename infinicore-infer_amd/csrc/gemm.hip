@@ -93,7 +93,13 @@ __device__ __forceinline__ void spread_token_operand(const v4s* glo, const v4s* 
     ((alo[Us][0] = row_from_above<(Us % AG) * MP>(glo[Us / AG]), ahi[Us][0] = row_from_above<(Us % AG) * MP>(ghi[Us / AG])), ...);
 }
 
-template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI, bool OWN_K = false, int AG = 1>
+// LINES (K a multiple of 64, aligned operands): the weights come in whole cache lines, a wave's load covering 8 rows x
+// 128 bytes (two k-steps), with the non-temporal hint: a kernel that only streams a weight matrix so takes 9.4 us for
+// the 2B shape's 53 MB gate/up matrix where loads in operand layout (16 rows x 64 bytes) take 15.6.  What a load
+// brings is not in operand layout, so each wave passes it through 2.3 KB of LDS of its own (rows 144 bytes apart: the
+// 16 rows of an operand read then fall into different banks) on its way to the matrix cores.
+constexpr int kLineRowBytes = 144;
+template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI, bool OWN_K = false, int AG = 1, bool LINES = false>
 __global__ void __launch_bounds__(WPB * 64)
 gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C,
                     int M, int N, int K, int lda, int ldw, int ldc, float alpha, RopeEpilogue rope, NormFuse nf) {
@@ -101,7 +107,11 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     constexpr bool CROPE = (EPI == 2);
     constexpr bool CRESID = (EPI == 3);
     constexpr int PV = kMaxSumParts / (WPB * 4);             // column-block sums a thread fetches
-    __shared__ float red[WPB - 1][NT * MT][64][4];
+    static_assert(!LINES || (ALIGNED && UNROLL % 2 == 0), "whole-line weight loads take k-steps in pairs");
+    // the waves' partial sums after the loop; while the loop runs the same memory passes the weights on (LINES)
+    constexpr int kRedBytes = (WPB - 1) * NT * MT * 64 * 4 * 4, kLineBytes = LINES ? WPB * 16 * kLineRowBytes : 0;
+    __shared__ __attribute__((aligned(16))) unsigned char red_mem[kRedBytes > kLineBytes ? kRedBytes : kLineBytes];
+    float (*red)[NT * MT][64][4] = reinterpret_cast<float (*)[NT * MT][64][4]>(red_mem);
     __shared__ float ssum[WPB * 4][16];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
@@ -147,6 +157,22 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         const int nrow = (base + r < lim) ? base + r : lim - 1;
         wp[nt] = W + (size_t)nrow * ldw + 8 * kq;
     }
+    // LINES: lane l loads 16 bytes of row 8 h + l / 8 of the tile (h = 0, 1) at byte 16 (l % 8) of a 128-byte line
+    const uint16_t* wp8[NT][2];
+    if (LINES) {
+#pragma unroll
+        for (int nt = 0; nt < NT; ++nt) {
+            int base = CSWIGLU ? n0 + 16 * (nt % G) + (nt / G) * NO : n0 + 16 * nt;
+            if (CROPE) base = n0 + nt * (rope_is_v ? rope.rr : (rope.dh >> 1));
+            const int lim = CSWIGLU ? (nt / G) * NO + sw_end : (CRESID ? rs_end : (CROPE ? base + rope.rr : N));
+#pragma unroll
+            for (int h = 0; h < 2; ++h) {
+                const int row = base + 8 * h + (lane >> 3);
+                wp8[nt][h] = W + (size_t)(row < lim ? row : lim - 1) * ldw + 8 * (lane & 7);
+            }
+        }
+    }
+    unsigned char* const line_buf = red_mem + (LINES ? wave * 16 * kLineRowBytes : 0);
     const uint16_t* ap[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -187,23 +213,42 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     const int s_begin = OWN_K ? wave * spw : wave;
     const int s_end = OWN_K ? ((wave + 1) * spw < nsteps ? (wave + 1) * spw : nsteps) : nsteps;
     constexpr int s_stride = OWN_K ? 1 : WPB;                // between the UNROLL steps of one iteration
-    for (int s0 = s_begin; s0 < s_end; s0 += s_stride * UNROLL) {
-        v4s wlo[UNROLL][NT], whi[UNROLL][NT], alo[UNROLL][MT], ahi[UNROLL][MT];
+    // LINES without OWN_K: the waves are dealt PAIRS of k-steps in turn (a 128-byte line holds two), and s0 counts pairs
+    constexpr bool PAIR_DEAL = LINES && !OWN_K;
+    auto step_at = [&](int s0, int u) { return PAIR_DEAL ? 2 * (s0 + (u >> 1) * WPB) + (u & 1) : s0 + u * s_stride; };
+    const int it_end = PAIR_DEAL ? (nsteps >> 1) : s_end;    // (K is a multiple of 64 with LINES: the steps come in whole pairs)
+    constexpr int it_stride = PAIR_DEAL ? WPB * (UNROLL / 2) : s_stride * UNROLL;
+    for (int s0 = s_begin; s0 < it_end; s0 += it_stride) {
+        v4s wlo[LINES ? 1 : UNROLL][NT], whi[LINES ? 1 : UNROLL][NT], alo[UNROLL][MT], ahi[UNROLL][MT];
+        uint4 wline[LINES ? UNROLL / 2 : 1][NT][2];
+        if constexpr (LINES) {
+#pragma unroll
+            for (int j = 0; j < UNROLL / 2; ++j) {
+                const int st = step_at(s0, 2 * j);
+                const bool ok = st < s_end;                  // (both steps of the pair exist, or neither)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt)
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        wline[j][nt][h] = ok ? load_stream16(wp8[nt][h] + 32 * st) : uint4{0, 0, 0, 0};
+            }
+        } else {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u) {
-            const int kk = 32 * (s0 + u * s_stride);
-            const int valid = (s0 + u * s_stride < s_end) ? K - kk - 8 * kq : 0;          // <= 0 beyond the end
+            const int kk = 32 * step_at(s0, u);
+            const int valid = (step_at(s0, u) < s_end) ? K - kk - 8 * kq : 0;          // <= 0 beyond the end
 #pragma unroll
             for (int nt = 0; nt < NT; ++nt) {
                 if (valid > 0) load8<ALIGNED>(wp[nt] + kk, valid, wlo[u][nt], whi[u][nt]);
                 else { wlo[u][nt] = v4s{0, 0, 0, 0}; whi[u][nt] = wlo[u][nt]; }
             }
         }
+        }
         if constexpr (AG == 1) {
 #pragma unroll
             for (int u = 0; u < UNROLL; ++u) {
-                const int kk = 32 * (s0 + u * s_stride);
-                const int valid = (s0 + u * s_stride < s_end) ? K - kk - 8 * kq : 0;
+                const int kk = 32 * step_at(s0, u);
+                const int valid = (step_at(s0, u) < s_end) ? K - kk - 8 * kq : 0;
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     if (valid > 0) load8<ALIGNED>(ap[mt] + kk, valid, alo[u][mt], ahi[u][mt]);
@@ -222,7 +267,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
             const uint16_t* gp = A + (size_t)((m0 + gm < M) ? m0 + gm : M - 1) * lda + 8 * kq;
 #pragma unroll
             for (int g = 0; g < UNROLL / AG; ++g) {
-                const int st = s0 + (g * AG + gt) * s_stride;
+                const int st = step_at(s0, g * AG + gt);
                 const int kk = 32 * st;
                 const int valid = (st < s_end && m0 + gm < M) ? K - kk - 8 * kq : 0;
                 if (valid > 0) load8<ALIGNED>(gp + kk, valid, glo[g], ghi[g]);
@@ -230,6 +275,33 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
             }
             spread_token_operand<AG, MP>(glo, ghi, alo, ahi, std::make_integer_sequence<int, UNROLL>{});
         }
+        typedef short v8s __attribute__((ext_vector_type(8)));
+        typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+        if constexpr (LINES) {
+#pragma unroll
+            for (int j = 0; j < UNROLL / 2; ++j)
+#pragma unroll
+                for (int nt = 0; nt < NT; ++nt) {
+                    // through this wave's LDS: in as rows of 128 bytes, out as the operands of the pair's two k-steps
+                    // (row r, bytes 16 kq .. of the first half and of the second).  LDS serves a wave's requests in order.
+#pragma unroll
+                    for (int h = 0; h < 2; ++h)
+                        *reinterpret_cast<uint4*>(line_buf + (8 * h + (lane >> 3)) * kLineRowBytes + 16 * (lane & 7)) = wline[j][nt][h];
+                    __builtin_amdgcn_wave_barrier();
+                    uint4 w2[2];
+#pragma unroll
+                    for (int e = 0; e < 2; ++e) w2[e] = *reinterpret_cast<const uint4*>(line_buf + r * kLineRowBytes + 16 * (4 * e + kq));
+                    __builtin_amdgcn_wave_barrier();
+#pragma unroll
+                    for (int e = 0; e < 2; ++e)
+#pragma unroll
+                        for (int mt = 0; mt < MT; ++mt) {
+                            const v8s a8 = __builtin_shufflevector(alo[2 * j + e][mt], ahi[2 * j + e][mt], 0, 1, 2, 3, 4, 5, 6, 7);
+                            acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w2[e]), __builtin_bit_cast(v8b, a8),
+                                                                                  acc[nt][mt], 0, 0, 0);
+                        }
+                }
+        } else {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
 #pragma unroll
@@ -237,14 +309,14 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
                 for (int mt = 0; mt < MT; ++mt) {
                     // one 16x16x32 product per k-step: a lane's 8 elements of W and of A are k = 8 kq .. 8 kq + 7 of the step
-                    typedef short v8s __attribute__((ext_vector_type(8)));
-                    typedef __bf16 v8b __attribute__((ext_vector_type(8)));
                     const v8s w8 = __builtin_shufflevector(wlo[u][nt], whi[u][nt], 0, 1, 2, 3, 4, 5, 6, 7);
                     const v8s a8 = __builtin_shufflevector(alo[u][mt], ahi[u][mt], 0, 1, 2, 3, 4, 5, 6, 7);
                     acc[nt][mt] = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w8), __builtin_bit_cast(v8b, a8),
                                                                           acc[nt][mt], 0, 0, 0);
                 }
+        }
     }
+    if (LINES) __syncthreads();                              // every wave is done passing weights through what now holds the sums
     if (wave > 0) {
 #pragma unroll
         for (int nt = 0; nt < NT; ++nt)
@@ -370,10 +442,22 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         }
 }
 
+// Whole-line weight loads (LINES) where the sizes allow: 1 (the default) on, 0 off (for measurements and tests).
+static int g_lines_enabled = 1;
+IC_EXPORT int ic_gemm_nt_lines_enable(int on) { g_lines_enabled = on ? 1 : 0; return IC_OK; }
+static inline bool lines_apply(bool aligned, int K) { return aligned && g_lines_enabled && K % 64 == 0; }
+
 template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0, bool OWN_K = false, int AG = 1>
 static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
                         int ldc, float alpha, bool aligned, const NormFuse& nf, hipStream_t stream, int blocks = 0) {
     dim3 grid(blocks > 0 ? blocks : (N + 16 * NT - 1) / (16 * NT), (M + 16 * MT - 1) / (16 * MT)), block(WPB * 64);
+    if constexpr (UNROLL % 2 == 0) {
+        if (lines_apply(aligned, K)) {
+            hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI, OWN_K, AG, true>), grid, block, 0, stream,
+                               (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
+            return;
+        }
+    }
     if (aligned)
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, NT, MT, WPB, UNROLL, true, EPI, OWN_K, AG>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, RopeEpilogue{}, nf);
@@ -390,6 +474,15 @@ static void launch_gemm_swiglu(const void* A, const void* W, void* C, int M, int
     if (blocks <= 0) blocks = (N / 2 + 16 * G - 1) / (16 * G);
     dim3 grid(blocks, (M + 15) / 16), block(WPB * 64);
     constexpr int AG = (UN % 4 == 0) ? 4 : 2;                // up to 4 rows one token load serves AG k-steps
+    if (lines_apply(aligned, K)) {
+        if (M <= 4 && sizeof(TC) == 2)
+            hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, true, 1, false, AG, true>), grid, block, 0, stream,
+                               (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
+        else
+            hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, true, 1, false, 1, true>), grid, block, 0, stream,
+                               (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
+        return;
+    }
     if (aligned && M <= 4 && sizeof(TC) == 2)
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<TC, 2 * G, 1, WPB, UN, true, 1, false, AG>), grid, block, 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, 1.0f, RopeEpilogue{}, nf);
@@ -780,7 +873,14 @@ IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int
     hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, WPB, UN, AL, 2>), grid, dim3(WPB * 64), 0, stream, \
                        (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf)
     // 8 waves, 4 steps in flight: within 4 % of the best tiling at every shape swept, and it does not spill
-    if (aligned && M <= 4)                                  // one token load serves the 4 k-steps of an iteration
+    if (lines_apply(aligned, K)) {
+        if (M <= 4)
+            hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, 8, 4, true, 2, false, 4, true>), grid, dim3(8 * 64), 0, stream,
+                               (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf);
+        else
+            hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, 8, 4, true, 2, false, 1, true>), grid, dim3(8 * 64), 0, stream,
+                               (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf);
+    } else if (aligned && M <= 4)                           // one token load serves the 4 k-steps of an iteration
         hipLaunchKernelGGL((gemm_nt_bf16_kernel<bf16, 2, 1, 8, 4, true, 2, false, 4>), grid, dim3(8 * 64), 0, stream,
                            (const uint16_t*)A, (const uint16_t*)W, (bf16*)C, M, N, K, lda, ldw, ldc, 1.0f, rope, nf);
     else if (aligned) IC_ROPE(8, 4, true);

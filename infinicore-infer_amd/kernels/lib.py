@@ -112,6 +112,7 @@ _SIGNATURES = {
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],
     "ic_gemm_nt_residual_parts": [_I],
     "ic_gemm_nt_wide_enable": [_I],
+    "ic_gemm_nt_lines_enable": [_I],
     "ic_peak_mfma_bf16": [_P, _I, _I, _P],
     "ic_peak_read": [_P, _LL, _I, _P, _P],
     "ic_gemm_nt_supported": [_I, _I, _I],
