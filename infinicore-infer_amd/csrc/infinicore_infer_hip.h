@@ -85,6 +85,9 @@ int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, 
 // Products of up to 16 rows with 32,768 weight rows or more (the output head) run in a kernel whose waves own whole
 // weight tiles; 0 sends them through the tiled kernel instead (for measurements).  Returns the previous setting.
 int ic_gemm_nt_wide_enable(int on);
+// 1 (the default): with K a multiple of 64 and aligned operands the few-row products read their weights in whole cache lines
+// (8 rows x 128 bytes a wave load, not kept in the caches) and pass them through LDS into operand layout; 0: loads in operand layout.
+int ic_gemm_nt_lines_enable(int on);
 // The same with the tiling chosen by the caller (tuning and tests); nt == 0 selects the SwiGLU variant.
 int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int nt, int wpb, int unroll, hipStream_t stream);
 // QKV projection of M <= 16 rows with rotary and cache write in the epilogue; row_factor nullable.

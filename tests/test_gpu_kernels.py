@@ -621,6 +621,52 @@ def test_norm_split_over_two_products(M, N, K, N2):
         _close(act, P.plain_swiglu(gu[:, :N2 // 2], gu[:, N2 // 2:]), torch.bfloat16, factor=2)
 
 
+@pytest.mark.parametrize("M", [1, 3, 8, 16])
+@pytest.mark.parametrize("N,K", [(331, 192), (2304, 2304), (1000, 1536), (512, 8192 + 64), (12000, 640)])
+def test_whole_line_weight_loads_equal_loads_in_operand_layout(M, N, K):
+    """With K a multiple of 64 the few-row products read their weights in whole cache lines and pass them through LDS;
+    switched off, the same entry points load in operand layout.  Both must give the plain product, the activation
+    epilogue and the residual epilogue alike (rows of 16 KB and more: a wave owns a run of k-steps)."""
+    from infinicore_infer_amd.kernels.lib import get_lib
+    ops, lib = _ops(), get_lib()
+    g = torch.Generator().manual_seed(61)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16)
+    x = torch.randn(M, N, generator=g)
+    gw = torch.rand(N, generator=g) + 0.5
+    ad, wd = a.to(DEV), w.to(DEV)
+    got = {}
+    try:
+        for on in (1, 0):
+            lib.ic_gemm_nt_lines_enable(on)
+            plain = torch.empty(M, N, dtype=torch.float32, device=DEV)
+            ops.gemm_nt(ad, wd, plain, 0.5)
+            res = None
+            if N % 2 == 0:
+                act = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+                ops.gemm_nt(ad, wd, act, swiglu_output=True)
+                xd = x.to(DEV)
+                y = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+                if ops.residual_parts(N) <= ops.MAX_SUMSQ_PARTS:
+                    sumsq = torch.zeros(ops.residual_parts(N), 16, device=DEV)
+                    ops.gemm_nt(ad, wd, y, residual=(xd, gw.to(DEV), 0.3, sumsq))
+                res = (act.float().cpu(), xd.cpu(), y.float().cpu())
+            got[on] = (plain.cpu(), res)
+    finally:
+        lib.ic_gemm_nt_lines_enable(1)
+    want = 0.5 * P.plain_linear(a, w)
+    for on in (1, 0):
+        _close(got[on][0], want, torch.float32, factor=20)
+    if got[1][1] is not None:
+        gu = P.round_bf16(P.plain_linear(a, w))
+        for on in (1, 0):
+            act, xs, y = got[on][1]
+            _close(act, P.plain_swiglu(gu[:, :N // 2], gu[:, N // 2:]), torch.bfloat16, factor=2)
+            if ops.residual_parts(N) <= ops.MAX_SUMSQ_PARTS:
+                _close(xs, x.double() + 0.3 * gu, torch.bfloat16, scale=0.3 * float(gu.abs().max()))
+                _close(y, xs.double() * gw.double(), torch.bfloat16)
+
+
 def test_gemm_qkv_rope_with_row_factors():
     g = torch.Generator().manual_seed(43)
     ops = _ops()
