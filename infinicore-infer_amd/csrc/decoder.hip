@@ -216,7 +216,9 @@ struct IcDecoder {
             const int* slots = b.group_slots[e.group];
             if (A.rot_dim > 0 && b.max_position >= A.max_positions) return fail(IC_ERR_ARG, "a position beyond the rotary tables", i);
             if (nkv > 0 && !slots) return fail(IC_ERR_ARG, "the cache slots of the entry's group", i);
-            const bool fused_qkv = few && nkv > 0 && A.rot_dim == A.head_dim && ic_gemm_qkv_rope_supported(IC_BF16, A.head_dim);
+            // (up to 16 rows, or up to 32 where the weights can be read in whole cache lines and no row factors are owed)
+            const bool fused_qkv = dt == IC_BF16 && nkv > 0 && A.rot_dim == A.head_dim && ic_gemm_qkv_rope_supported(IC_BF16, A.head_dim) &&
+                                   (few || (!h_def && T <= ic_gemm_nt_epilogue_rows(2, d, d, d)));
             IcRowFactor rf{};
             if (h_def) rf = IcRowFactor{h_def->sumsq, h_def->parts, h_def->width, h_def->eps};
             if (fused_qkv) {
@@ -292,7 +294,7 @@ struct IcDecoder {
             // ---- feed-forward ----------------------------------------------------------------------------------
             const int di = L.ffn.intermediate;
             void* act = base + ws.act;
-            if (few) {
+            if (few || (dt == IC_BF16 && !g_def && T <= ic_gemm_nt_epilogue_rows(1, d, d, d))) {      // (up to 32 rows with whole-line loads)
                 IcRowFactor gf{};
                 if (g_def) gf = IcRowFactor{g_def->sumsq, g_def->parts, g_def->width, g_def->eps};
                 st = ic_gemm_nt(g, IC_BF16, L.ffn.w_gate_up, IC_BF16, act, IC_BF16, T, 2 * di, d, d, d, di, 1.0f, 1, g_def ? &gf : nullptr,

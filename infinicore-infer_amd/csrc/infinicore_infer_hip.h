@@ -88,6 +88,9 @@ int ic_gemm_nt_wide_enable(int on);
 // 1 (the default): with K a multiple of 64 and aligned operands the few-row products read their weights in whole cache lines
 // (8 rows x 128 bytes a wave load, not kept in the caches) and pass them through LDS into operand layout; 0: loads in operand layout.
 int ic_gemm_nt_lines_enable(int on);
+// Rows that the products with an epilogue take: kind 1 (c_mode 1, SwiGLU) and kind 2 (ic_gemm_qkv_rope) 32 where the weights can be
+// read in whole cache lines (K a multiple of 64, row strides multiples of 8), 16 otherwise; without row factors above 16 rows.
+int ic_gemm_nt_epilogue_rows(int kind, int K, int lda, int ldw);
 // The same with the tiling chosen by the caller (tuning and tests); nt == 0 selects the SwiGLU variant.
 int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int nt, int wpb, int unroll, hipStream_t stream);
 // QKV projection of M <= 16 rows with rotary and cache write in the epilogue; row_factor nullable.

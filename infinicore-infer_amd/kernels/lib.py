@@ -113,6 +113,7 @@ _SIGNATURES = {
     "ic_gemm_nt_residual_parts": [_I],
     "ic_gemm_nt_wide_enable": [_I],
     "ic_gemm_nt_lines_enable": [_I],
+    "ic_gemm_nt_epilogue_rows": [_I, _I, _I, _I],
     "ic_peak_mfma_bf16": [_P, _I, _I, _P],
     "ic_peak_read": [_P, _LL, _I, _P, _P],
     "ic_gemm_nt_supported": [_I, _I, _I],

@@ -359,9 +359,15 @@ def _row_factor(row_factor, M, what):
     return IcRowFactor(sumsq.data_ptr(), sumsq.shape[0], int(width), float(eps))
 
 
+def gemm_epilogue_rows(kind: str, a, w) -> int:
+    """Rows that the product with the ``kind`` epilogue ("swiglu", or "rope" for gemm_qkv_rope) takes for these operands: 32
+    where the weights can be read in whole cache lines, 16 otherwise (and above 16 rows without row factors)."""
+    return int(get_lib().ic_gemm_nt_epilogue_rows({"swiglu": 1, "rope": 2}[kind], int(a.shape[1]), int(a.stride(0)), int(w.stride(0))))
+
+
 def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_factor=None, residual=None):
     """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation).
-    swiglu_output (M <= 16): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate).
+    swiglu_output (M <= gemm_epilogue_rows("swiglu", a, w)): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate).
     row_factor = (sumsq [n_parts, 16], width, eps), M <= 16: row m of the product is first multiplied by
     rsqrt(sumsq[:, m].sum() / width + eps), the factor an RMS norm of a's rows still owes.
     residual = (x float32 [M, N], weight float32 [N], beta, sumsq_out float32 [residual_parts(N), 16]),
@@ -372,7 +378,7 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
     M, K = a.shape
     N = w.shape[0]
     _need(w.shape[1] == K and tuple(out.shape) == (M, N // 2 if swiglu_output else N), "gemm_nt: shape mismatch")
-    _need(not swiglu_output or (M <= 16 and N % 2 == 0), "gemm_nt: fused activation needs M <= 16 and even N")
+    _need(not swiglu_output or (M <= 32 and N % 2 == 0), "gemm_nt: fused activation needs M <= 32 and even N")
     _need(a.stride(1) == 1 and w.stride(1) == 1 and out.stride(1) == 1, "gemm_nt: inner strides must be 1")
     rf = _row_factor(row_factor, M, "gemm_nt")
     rn = None
@@ -502,7 +508,7 @@ def gemm_qkv_rope_tile_rows(rows: int) -> None:
 
 def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads, n_kv_heads, head_dim, page_size,
                   row_factor=None):
-    """For M <= 16 rows: qkv = a @ w^T with the rotary encoding and the cache write in the epilogue.
+    """For M <= gemm_epilogue_rows("rope", a, w) rows: qkv = a @ w^T with the rotary encoding and the cache write in the epilogue.
     The q heads of qkv[M, >= n_heads * head_dim] hold rotated queries afterwards; rotated keys and
     the values are in cache slot ``slots[m]``.  Full rotary, bfloat16.  row_factor: as in gemm_nt."""
     import ctypes
@@ -510,7 +516,7 @@ def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads
     M, K = a.shape
     _i32(positions, "positions")
     _i32(slots, "slots")
-    _need(M <= 16 and positions.numel() == M and slots.numel() == M, "gemm_qkv_rope: at most 16 rows, one position and slot each")
+    _need(M <= 32 and positions.numel() == M and slots.numel() == M, "gemm_qkv_rope: at most 32 rows, one position and slot each")
     rf = _row_factor(row_factor, M, "gemm_qkv_rope")
     _need(tuple(w.shape) == ((n_heads + 2 * n_kv_heads) * head_dim, K), "gemm_qkv_rope: weight shape")
     _need(qkv.shape[0] == M and qkv.shape[1] >= n_heads * head_dim and qkv.stride(1) == 1

@@ -93,9 +93,12 @@ class Rotary(PositionEncoding):
         row_factor = None
         if isinstance(h, DeferredRows):
             h, row_factor = h.values, h.row_factor()
-        if (h.shape[0] > FEW_ROWS or rt.gemm_impl != "auto" or n_kv_heads == 0 or self.rot_dim != head_dim
+        if (rt.gemm_impl != "auto" or n_kv_heads == 0 or self.rot_dim != head_dim
                 or h.dtype != torch.bfloat16 or w_qkv.dtype != torch.bfloat16
                 or not ops.gemm_qkv_rope_supported(h.dtype, head_dim)):
+            return False
+        # up to 16 rows, or as many as the kernel takes with whole-line weight loads when no row factors are owed
+        if h.shape[0] > FEW_ROWS and (row_factor is not None or h.shape[0] > ops.gemm_epilogue_rows("rope", h, w_qkv)):
             return False
         if ctx.max_position >= self.max_positions:
             raise ValueError("position %d is beyond the rotary tables (%d)" % (ctx.max_position, self.max_positions))

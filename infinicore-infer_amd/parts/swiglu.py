@@ -58,7 +58,10 @@ class SwiGLU(FeedForward):
         rt = self.runtime
         T = h.shape[0]
         act = ctx.ws.buffer("ffn_act", (T, self.intermediate_size), rt.dtype)
-        if own_kernel_applies(T, h.dtype, self.w_gate_up.dtype, act.dtype, rt.gemm_impl):
+        few = own_kernel_applies(T, h.dtype, self.w_gate_up.dtype, act.dtype, rt.gemm_impl)
+        if not few and not isinstance(h, DeferredRows) and own_kernel_applies(1, h.dtype, self.w_gate_up.dtype, act.dtype, rt.gemm_impl):
+            few = T <= ops.gemm_epilogue_rows("swiglu", h, self.w_gate_up)      # up to 32 rows with whole-line weight loads
+        if few:
             # few rows: the activation is the epilogue of the gate/up projection
             if isinstance(h, DeferredRows):
                 ops.gemm_nt(h.values, self.w_gate_up, act, swiglu_output=True, row_factor=h.row_factor())

@@ -521,7 +521,8 @@ def test_sampling_distribution():
 
 @pytest.mark.parametrize("cdtype", DT)
 @pytest.mark.parametrize("M,di,K", [(1, 344, 200), (8, 5760, 2304), (16, 256, 96), (5, 130, 100), (3, 3840, 1536),
-                                    (5, 8400, 136), (2, 8400, 2048)])    # the last two: more tiles than one round of blocks takes
+                                    (5, 8400, 136), (2, 8400, 2048),     # the last two: more tiles than one round of blocks takes
+                                    (17, 5760, 2304), (32, 3840, 1536), (25, 344, 192), (31, 16384, 128)])   # 17..32 rows: two row tiles
 def test_gemm_nt_with_swiglu_output(cdtype, M, di, K):
     """The gate/up projection with the activation in its epilogue equals the plain product
     followed by the SwiGLU kernel."""
@@ -529,6 +530,11 @@ def test_gemm_nt_with_swiglu_output(cdtype, M, di, K):
     h = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (torch.randn(2 * di, K, generator=g) * 0.1).to(torch.bfloat16)
     out = torch.empty(M, di, dtype=cdtype, device=DEV)
+    if M > 16 and cdtype != torch.bfloat16:          # two row tiles exist for bfloat16 results only: refused, not computed wrongly
+        with pytest.raises(_ops().KernelError):
+            _ops().gemm_nt(h.to(DEV), w.to(DEV), out, swiglu_output=True)
+        return
+    assert M <= _ops().gemm_epilogue_rows("swiglu", h, w)
     _ops().gemm_nt(h.to(DEV), w.to(DEV), out, swiglu_output=True)
     rnd = P.round_bf16 if cdtype == torch.bfloat16 else (lambda t: t)
     gu = rnd(P.plain_linear(h, w))
@@ -536,7 +542,10 @@ def test_gemm_nt_with_swiglu_output(cdtype, M, di, K):
 
 
 @pytest.mark.parametrize("M,nh,nkvh,dh,K,page", [(1, 4, 2, 32, 96, 16), (8, 6, 2, 64, 200, 16), (16, 3, 3, 64, 2304, 64),
-                                                 (5, 4, 1, 128, 344, 32), (3, 36, 36, 64, 2304, 64)])
+                                                 (5, 4, 1, 128, 344, 32), (3, 36, 36, 64, 2304, 64),
+                                                 # 17..32 rows: two row tiles per block (whole-line weight loads)
+                                                 (17, 6, 2, 64, 1536, 64), (32, 3, 3, 64, 2304, 16), (25, 4, 1, 128, 640, 32),
+                                                 (20, 5, 5, 32, 192, 16), (31, 36, 36, 64, 2304, 64)])
 @pytest.mark.parametrize("tile_rows", [0, 16, 8, 4])
 def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page, tile_rows):
     """The fused projection + rotary + cache write equals the plain product followed by the
