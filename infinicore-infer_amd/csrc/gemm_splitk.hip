@@ -39,6 +39,10 @@ __global__ void __launch_bounds__(kSkThreads)
 gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, float* __restrict__ P,
                    int M, int N, int K, int lda, int ldw, int chunks_per_slice, int rotate) {
     __shared__ __attribute__((aligned(16))) unsigned char a_lds[2][16 * MT][kSkRowBytes];
+    // The weights come in whole cache lines, a wave's load covering 8 rows x 128 bytes with the non-temporal hint (a stream
+    // of such loads runs a third faster than one of loads in operand layout, 16 rows x 64 bytes), and pass through
+    // this wave-private tile on their way into operand layout (LDS serves a wave's requests in order: no barrier).
+    __shared__ __attribute__((aligned(16))) unsigned char w_lds[kSkThreads / 64][16][kSkRowBytes];
     const int tid = threadIdx.x, lane = tid & 63, wave = tid >> 6;
     const int r = lane & 15, kq = lane >> 4;
     const int n0 = blockIdx.x * kSkCols + 16 * wave;
@@ -60,8 +64,13 @@ gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
     };
 
     // this lane's weight row (clamped: rows beyond N repeat the last one and are not stored)
-    const int nrow = (n0 + r < N) ? n0 + r : N - 1;
-    const uint16_t* wp = W + (size_t)nrow * ldw + 8 * kq;
+    // load i of a chunk: rows 8 (i % 2) + lane / 8 of the wave's 16, bytes 128 (i / 2) + 16 (lane % 8) of the chunk's 256
+    const uint16_t* wp8[2];
+#pragma unroll
+    for (int h = 0; h < 2; ++h) {
+        const int row = n0 + 8 * h + (lane >> 3);
+        wp8[h] = W + (size_t)(row < N ? row : N - 1) * ldw + 8 * (lane & 7);
+    }
     // the A pieces this thread brings into LDS: piece p = tid + 256 i is row p / 16, bytes 16 (p % 16) of the chunk
     const uint16_t* ap[MT];
     int a_row[MT], a_col[MT];
@@ -94,8 +103,9 @@ gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
         const int k0 = k_of(c);
 #pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const bool ok = c < c_end && k0 + 32 * u + 8 * kq + 8 <= K;
-            wreg[J][u] = ld16(wp + (ok ? k0 + 32 * u : 0));
+            const int k = k0 + 64 * (u >> 1);
+            const bool ok = c < c_end && k + 8 * (lane & 7) + 8 <= K;
+            wreg[J][u] = load_stream16(wp8[u & 1] + (ok ? k : 0));
         }
     };
     auto fetch_a = [&](int c, auto set) {
@@ -120,8 +130,16 @@ gemm_splitk_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ 
     auto multiply = [&](auto wset, auto stage) {
         constexpr int J = decltype(wset)::value, L = decltype(stage)::value;
 #pragma unroll
+        for (int u = 0; u < 4; ++u)
+            *reinterpret_cast<uint4*>(&w_lds[wave][8 * (u & 1) + (lane >> 3)][128 * (u >> 1) + 16 * (lane & 7)]) = wreg[J][u];
+        __builtin_amdgcn_wave_barrier();
+        uint4 wop[4];
+#pragma unroll
+        for (int u = 0; u < 4; ++u) wop[u] = *reinterpret_cast<const uint4*>(&w_lds[wave][r][64 * u + 16 * kq]);
+        __builtin_amdgcn_wave_barrier();
+#pragma unroll
         for (int u = 0; u < 4; ++u) {
-            const sk_v8b w8 = __builtin_bit_cast(sk_v8b, wreg[J][u]);
+            const sk_v8b w8 = __builtin_bit_cast(sk_v8b, wop[u]);
 #pragma unroll
             for (int mt = 0; mt < MT; ++mt) {
                 const uint4 a = *reinterpret_cast<const uint4*>(&a_lds[L][16 * mt + r][2 * (32 * u + 8 * kq)]);
