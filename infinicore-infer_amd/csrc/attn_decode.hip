@@ -391,39 +391,34 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
         for (int c = 0; c < ND; ++c) oacc[c] = gq_v4f{0.f, 0.f, 0.f, 0.f};
         float m = -INFINITY, l = 0.f;              // of head lr, the same in the four lane groups
 
+        // Keys and values are read in whole rows (consecutive lanes take consecutive 16-byte pieces, so a wave's load
+        // covers whole cache lines) with loads the caches do not keep.  The keys then pass through the wave's LDS tile
+        // into operand layout (key 16 s2 + lr, dims 32 c + 8 lg .. +7) before the values take the tile over: loaded
+        // straight in operand layout a wave's load covered 64 bytes of each of 16 rows, half a line.
         GqFrag kreg[2][NC];
-        uint4 vreg[NV];
+        uint4 kraw[NV], vreg[NV];
         auto fetch = [&](int tile) {
             const int kt = lo + tile * kGqaKeys;
-#pragma unroll
-            for (int s2 = 0; s2 < 2; ++s2) {
-                const int key = kt + 16 * s2 + lr;
-                const bool ok = tile < n_tiles && key < hi;
-                const size_t off = ok ? row_of(key) + 8 * lg : 0;
-#pragma unroll
-                for (int c = 0; c < NC; ++c) {
-                    // (plain loads: a wave's load covers 64 bytes of each of 16 key rows, half a cache line, and the other
-                    // half comes with the next load; without the caches keeping the line it would be fetched twice.
-                    // The values below and both planes in the kernel above are read in whole rows and are streamed.)
-                    if (ok) kreg[s2][c].u = *reinterpret_cast<const uint4*>(kbase + off + 32 * c);
-                    else kreg[s2][c].u = make_uint4(0, 0, 0, 0);
-                }
-            }
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int idx = lane + 64 * i;
                 const int vkey = idx / (DH / 8), oct = idx - vkey * (DH / 8);
                 const int key = kt + vkey;
+                kraw[i] = make_uint4(0, 0, 0, 0);
                 vreg[i] = make_uint4(0, 0, 0, 0);
-                if (tile < n_tiles && key < hi) vreg[i] = load_stream16(vbase + row_of(key) + oct * 8);
+                if (tile < n_tiles && key < hi) {
+                    const size_t at = row_of(key) + oct * 8;
+                    kraw[i] = load_stream16(kbase + at);
+                    vreg[i] = load_stream16(vbase + at);
+                }
             }
         };
-        auto stash = [&]() {
+        auto stash = [&](const uint4* regs) {
 #pragma unroll
             for (int i = 0; i < NV; ++i) {
                 const int idx = lane + 64 * i;
                 const int vkey = idx / (DH / 8), oct = idx - vkey * (DH / 8);
-                *reinterpret_cast<uint4*>(&Vs[wave][vkey * VS + oct * 8]) = vreg[i];
+                *reinterpret_cast<uint4*>(&Vs[wave][vkey * VS + oct * 8]) = regs[i];
             }
         };
 
@@ -436,7 +431,15 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
             if (tile >= n_tiles) break;             // uniform in the wave
             const int kt = lo + tile * kGqaKeys;
             __builtin_amdgcn_wave_barrier();
-            stash();
+            stash(kraw);
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int s2 = 0; s2 < 2; ++s2)
+#pragma unroll
+                for (int c = 0; c < NC; ++c)
+                    kreg[s2][c].u = *reinterpret_cast<const uint4*>(&Vs[wave][(16 * s2 + lr) * VS + 32 * c + 8 * lg]);
+            __builtin_amdgcn_wave_barrier();
+            stash(vreg);
             __builtin_amdgcn_wave_barrier();
 
             // ---- S^T = K Q^T, two subtiles of 16 keys ----------------------------------
