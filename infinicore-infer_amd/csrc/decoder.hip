@@ -109,12 +109,11 @@ struct IcDecoder {
         w.part_acc = take(acc * 4);
         w.part_ml = take(ml * 4);
         w.head_in = take((size_t)b.n_want * d * ds);
-        size_t slices = 0;           // the O and down products of 17..64 rows as slices over K
-        if (meta.dtype == IC_BF16 && T > kFewRows && T <= kMidRows)
-            for (const IcLayer& l : layers) {
-                slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, l.attention.n_heads * l.attention.head_dim));
-                slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, l.ffn.intermediate));
-            }
+        size_t slices = 0;           // the O and down products as slices over K, where that pays
+        if (meta.dtype == IC_BF16 && T <= kMidRows)
+            for (const IcLayer& l : layers)
+                for (const int K : {l.attention.n_heads * l.attention.head_dim, l.ffn.intermediate})
+                    if (ic_gemm_splitk_pays(T, meta.hidden, K)) slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, K));
         w.tail_parts = take(slices * T * d * 4);
         size_t cut = 0;              // the states of prompt tiles whose walk over the keys is cut into parts
         if (meta.dtype == IC_BF16 && b.n_prefill_tiles > 0)
@@ -140,13 +139,13 @@ struct IcDecoder {
         return ic_matmul(a, meta.dtype, w, out, out_dtype, M, N, K, lda, K, N, alpha, lib_ws, lib_ws_bytes, stream);
     }
 
-    // 17..64 rows into the residual stream: x += alpha * (a w^T), out = rmsnorm(x) * weight, through the sliced
+    // 17..64 rows (and 13..16 long ones) into the residual stream: x += alpha * (a w^T), out = rmsnorm(x) * weight, through the sliced
     // product when it pays.  Returns 1 when done, 0 when the caller has to take the other way, < 0 on a fault.
     int tail_in_slices(const void* a, int K, const void* w, float* parts, float* x, float alpha, const float* weight, float eps,
                        void* out, int T, hipStream_t stream, int* status) const {
         const int d = meta.hidden;
         *status = IC_OK;
-        if (meta.dtype != IC_BF16 || T <= kFewRows || T > kMidRows || d % 4 || !ic_gemm_splitk_supported(T, d, K, K, K) ||
+        if (meta.dtype != IC_BF16 || T > kMidRows || d % 4 || !ic_gemm_splitk_supported(T, d, K, K, K) ||
             !ic_gemm_splitk_pays(T, d, K))
             return 0;
         const int slices = ic_gemm_splitk_slices(d, K);

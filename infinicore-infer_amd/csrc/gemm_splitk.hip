@@ -300,8 +300,16 @@ IC_EXPORT int ic_gemm_splitk_slices(int N, int K) {
 }
 
 // 1 when the sliced product is the faster way for this product: enough blocks to occupy half the chip.
+// Up to 16 rows the few-row product with the residual add in its epilogue is the faster one, but for 13..16 rows of
+// 16 KB and more (from 9 rows on it loads its token operand once per k-step: the 8B shape's down projection takes 34 us
+// at 16 rows, the slices and the kernel that sums them 27.5; a decode step of that shape 4.06 -> 3.95 ms at batch 16,
+// 3.76 -> 3.76 at 12, 3.64 -> 3.69 at 9).
+static int g_sk_few_rows = 1;
+// For measurements: 0 leaves products of up to 16 rows to the few-row kernel throughout.
+IC_EXPORT int ic_gemm_splitk_few_rows(int on) { const int was = g_sk_few_rows; g_sk_few_rows = on != 0; return was; }
 IC_EXPORT int ic_gemm_splitk_pays(int M, int N, int K) {
-    if (M <= 16 || M > 64 || N <= 0 || K <= 0 || N > 8192) return 0;
+    if (M <= 0 || M > 64 || N <= 0 || K <= 0 || N > 8192) return 0;
+    if (M <= 16 && (M <= 12 || K < 8192 || !g_sk_few_rows)) return 0;
     const int col_blocks = (N + kSkCols - 1) / kSkCols;
     return 2 * col_blocks * ic_gemm_splitk_slices(N, K) >= compute_units_sk();
 }

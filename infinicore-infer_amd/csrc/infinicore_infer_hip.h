@@ -107,6 +107,7 @@ int ic_gemm_splitk_supported(int M, int N, int K, int lda, int ldw);
 int ic_gemm_splitk_slices(int N, int K);      // how many slices to use (never an empty one)
 int ic_gemm_splitk_pays(int M, int N, int K);
 int ic_gemm_splitk_rotate(int on);            // for measurements: 0 = every block walks its slice of K from the start (default 1: rotated starts)
+int ic_gemm_splitk_few_rows(int on);          // for measurements: 0 = products of up to 16 rows never run in slices (default 1: 13..16 rows of 16 KB and more do)
 int ic_gemm_splitk(const void* A, const void* W, float* P, int M, int N, int K, int lda, int ldw, int n_slices, hipStream_t stream);
 // P [S, M, d]: x += alpha * (the product, rounded to bfloat16); out = rmsnorm(x) * w.
 int ic_splitk_add_rmsnorm(const float* P, int n_slices, int M, float* x, float alpha, const float* w, void* out, int d, float eps, hipStream_t stream);

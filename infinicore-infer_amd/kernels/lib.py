@@ -130,6 +130,7 @@ _SIGNATURES = {
     "ic_gemm_splitk": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "ic_gemm_splitk_pays": [_I, _I, _I],
     "ic_gemm_splitk_rotate": [_I],
+    "ic_gemm_splitk_few_rows": [_I],
     "ic_splitk_add_rmsnorm": [_P, _I, _I, _P, _F, _P, _P, _I, _F, _P],
     "ic_decoder_create": [_c.POINTER(IcDecoderMeta), _c.POINTER(IcLayer), _c.POINTER(IcRunEntry)],
     "ic_decoder_create_error": [],

@@ -78,10 +78,10 @@ def linear_tail(x, w, tail, ws, name: str, impl: str = "auto"):
     M, N = x.shape[0], w.shape[0]
     if tail is None:
         return None
-    if (impl == "auto" and FEW_ROWS < M <= MID_ROWS and tuple(tail.x.shape) == (M, N) and N % 4 == 0
+    if (impl == "auto" and M <= MID_ROWS and tuple(tail.x.shape) == (M, N) and N % 4 == 0
             and ops.gemm_splitk_supported(x, w) and ops.gemm_splitk_pays(M, N, w.shape[1])):
-        # 17..64 rows into the residual stream: the product as slices over K; the kernel that sums them does
-        # the add and the whole norm, so the rows handed on owe nothing
+        # 17..64 rows into the residual stream (and 13..16 long ones): the product as slices over K; the kernel that
+        # sums them does the add and the whole norm, so the rows handed on owe nothing
         slices = ops.gemm_splitk_slices(N, w.shape[1])
         parts = ops.gemm_splitk(x, w, ws.buffer("tail_parts", (slices * M * N,), torch.float32), slices)
         y = ws.buffer(name + "_values", (M, N), torch.bfloat16)

@@ -132,6 +132,38 @@ def test_decoding_twenty_requests_at_once(tmp_path_factory, name, dname, dtype, 
     engine.cache.check_invariants()
 
 
+@pytest.mark.parametrize("native", [True, False])
+def test_fourteen_rows_of_16_kb_go_through_the_sliced_product(tmp_path_factory, native):
+    """13..16 rows whose down projection reads rows of 16 KB (intermediate 8,192): that product runs as slices over K with
+    the kernel that sums them, adds the residual and norms, while the O projection (rows of 2 KB) keeps the few-row
+    kernel with the norm split over two products.  Fourteen requests decode together, bfloat16, against the plain model."""
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.kernels import ops
+    from infinicore_infer_amd.weights import write_random_model
+    import os
+    cfg = dict(model_type="minicpm", vocab_size=1003, hidden_size=1024, num_hidden_layers=2, num_attention_heads=8,
+               num_key_value_heads=2, intermediate_size=8192, max_position_embeddings=256, rms_norm_eps=1e-5,
+               rope_theta=10000.0, scale_emb=4, dim_model_base=256, scale_depth=1.4, tie_word_embeddings=False, eos_token_id=2)
+    assert ops.gemm_splitk_pays(14, 1024, 8192) and not ops.gemm_splitk_pays(14, 1024, 1024) and not ops.gemm_splitk_pays(12, 1024, 8192)
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "model_long_rows")
+    if not os.path.exists(os.path.join(folder, "model.safetensors")):
+        write_random_model(folder, cfg, seed=21, std=0.02)
+    n_req, n_dec = 14, 4
+    lens = [2 + (5 * i) % 23 for i in range(n_req)]
+    requests = {"s%d" % i: H.random_tokens(cfg["vocab_size"], lens[i] + n_dec, 900 + i) for i in range(n_req)}
+    steps = [{"step": 0, "end": [],
+              "entries": [{"id": k, "tokens": t[:lens[i]], "want": [lens[i] - 1]} for i, (k, t) in enumerate(requests.items())]}]
+    for j in range(n_dec):
+        steps.append({"step": j + 1, "end": list(requests) if j == n_dec - 1 else [],
+                      "entries": [{"id": k, "tokens": [t[lens[i] + j]], "want": [0]} for i, (k, t) in enumerate(requests.items())]})
+    engine = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=n_req * 64, page_size=16, max_requests=n_req, use_native=native)
+    got = H.run_trace(engine, steps)
+    ref = H.plain_logits(cfg, H.load_state_dict(folder), requests, True)
+    assert len(got) == n_req * (1 + n_dec)
+    H.compare(got, ref, H.BF16_TOL, "fourteen requests, long rows, native %s" % native)
+    engine.cache.check_invariants()
+
+
 def test_out_of_pages_changes_nothing(tmp_path_factory):
     from infinicore_infer_amd.cache import OutOfPages
     from infinicore_infer_amd.engine import StepEntry
