@@ -526,11 +526,16 @@ static int compute_units() {
 // before the current group is used, so its weight stream never pauses between tiles.  A block owns a run of whole
 // tiles and its waves equal shares of the run's (tile, group) pairs, so that every wave reads the same number of
 // bytes; where a share ends inside a tile, the two waves that hold the tile's halves add them through LDS.
+// LINES: the weights come in whole cache lines as in the tiled kernel (a wave load covers 8 rows x 128 bytes, not kept
+// in the caches) and pass through 2.3 KB of LDS of the wave's own into operand layout.  Alone, cold, 1 / 8 / 16 rows, a
+// float32 result: 122,753 x 2,304 107 / 114 / 122 -> 95 / 101 / 107 us, 73,448 x 4,096 109 / 113 / 116 -> 101 / 101 / 104;
+// 73,448 x 1,536 44.5 / 45.9 / 47.8 -> 46.6 / 47.4 / 49.8 (slower), and rows that do not start on a line (50,001 x 1,000)
+// 27 -> 36: the launcher takes this way for rows of 4 KB and more that are whole lines.
 constexpr int kWideDepth = 8;
 constexpr int kWideLdsLimit = 160 * 1024;             // LDS of a compute unit
 
 // WV waves a block: 8 when two blocks' token rows fit a compute unit's LDS, else 16 in one block
-template <typename TC, int WV>
+template <typename TC, int WV, bool LINES>
 __global__ void __launch_bounds__(WV * 64)
 gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W, TC* __restrict__ C, int M, int N, int K,
                  int lda, int ldw, int ldc, float alpha, NormFuse nf, int a_stride) {
@@ -538,7 +543,10 @@ gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
     uint16_t* As = reinterpret_cast<uint16_t*>(wide_smem);                       // [M][a_stride]
     float* part = reinterpret_cast<float*>(wide_smem + (size_t)M * a_stride * 2);    // [4 WV][16]
     float* rowf_s = part + 4 * WV * 16;                                          // [16]
-    v4f* heads = reinterpret_cast<v4f*>(rowf_s + 16);                            // [WV][64]
+    // per wave: after the loop the wave's unfinished tile lies here for its neighbour; LINES: during the loop 16 rows of
+    // 128 bytes, kLineRowBytes apart, that pass the weights on
+    constexpr int kWaveBuf = LINES ? 16 * kLineRowBytes : 64 * 16;
+    unsigned char* const line_buf = reinterpret_cast<unsigned char*>(rowf_s + 16) + (size_t)(threadIdx.x >> 6) * kWaveBuf;
     const int tid = threadIdx.x, lane = tid & 63, r = lane & 15, kq = lane >> 4;
     const int wave = __builtin_amdgcn_readfirstlane(tid >> 6);
     constexpr int D = kWideDepth;
@@ -550,15 +558,30 @@ gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
     const int klast = K - 8;                                 // the last whole 16 bytes of a weight row
     // group L of this wave's run (clamped to its last one, so that loads are never conditional): weights only;
     // columns beyond K repeat the row's last 16 bytes and meet zeros of the staged token rows
+    // LINES: w[2 j + h]: lane l holds 16 bytes of row 8 h + l / 8 of the tile, at byte 16 (l % 8) of the 128 that k-steps
+    // 2 j and 2 j + 1 of the group cover; else w[u] is the lane's operand of k-step u
     auto issue = [&](uint4 (&w)[D], int L) {
         L = run0 + (L < total ? L : total - 1);
         const int ti = L / groups, g = L - ti * groups;
-        const int n = (t0 + ti) * 16 + r;
-        const uint16_t* p = W + (size_t)(n < N ? n : N - 1) * ldw;
+        if constexpr (!LINES) {
+            const int n = (t0 + ti) * 16 + r;
+            const uint16_t* p = W + (size_t)(n < N ? n : N - 1) * ldw;
 #pragma unroll
-        for (int u = 0; u < D; ++u) {
-            const int k = 32 * (g * D + u) + 8 * kq;
-            w[u] = *reinterpret_cast<const uint4*>(p + (k < klast ? k : klast));
+            for (int u = 0; u < D; ++u) {
+                const int k = 32 * (g * D + u) + 8 * kq;
+                w[u] = *reinterpret_cast<const uint4*>(p + (k < klast ? k : klast));
+            }
+            return;
+        }
+#pragma unroll
+        for (int h = 0; h < 2; ++h) {
+            const int n = (t0 + ti) * 16 + 8 * h + (lane >> 3);
+            const uint16_t* p = W + (size_t)(n < N ? n : N - 1) * ldw;
+#pragma unroll
+            for (int j = 0; j < D / 2; ++j) {
+                const int k = 32 * (g * D + 2 * j) + 8 * (lane & 7);
+                w[2 * j + h] = load_stream16(p + (k < klast ? k : klast));
+            }
         }
     };
     uint4 w0[D], w1[D];
@@ -617,10 +640,30 @@ gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
     bool in_tail = has_tail;
     auto use = [&](const uint4 (&w)[D]) {
         typedef __bf16 v8b __attribute__((ext_vector_type(8)));
+        if constexpr (!LINES) {
 #pragma unroll
-        for (int u = 0; u < D; ++u) {
-            const uint4 a = *reinterpret_cast<const uint4*>(arow + 32 * (cg * D + u));
-            acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w[u]), __builtin_bit_cast(v8b, a), acc, 0, 0, 0);
+            for (int u = 0; u < D; ++u) {
+                const uint4 a = *reinterpret_cast<const uint4*>(arow + 32 * (cg * D + u));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w[u]), __builtin_bit_cast(v8b, a), acc, 0, 0, 0);
+            }
+        } else {
+#pragma unroll
+        for (int j = 0; j < D / 2; ++j) {
+            // in as rows of 128 bytes, out as the operands of the pair's two k-steps; LDS serves a wave's requests in order
+#pragma unroll
+            for (int h = 0; h < 2; ++h)
+                *reinterpret_cast<uint4*>(line_buf + (8 * h + (lane >> 3)) * kLineRowBytes + 16 * (lane & 7)) = w[2 * j + h];
+            __builtin_amdgcn_wave_barrier();
+            uint4 w2[2];
+#pragma unroll
+            for (int e = 0; e < 2; ++e) w2[e] = *reinterpret_cast<const uint4*>(line_buf + r * kLineRowBytes + 16 * (4 * e + kq));
+            __builtin_amdgcn_wave_barrier();
+#pragma unroll
+            for (int e = 0; e < 2; ++e) {
+                const uint4 a = *reinterpret_cast<const uint4*>(arow + 32 * (cg * D + 2 * j + e));
+                acc = __builtin_amdgcn_mfma_f32_16x16x32_bf16(__builtin_bit_cast(v8b, w2[e]), __builtin_bit_cast(v8b, a), acc, 0, 0, 0);
+            }
+        }
         }
         if (++cg == groups) {
             if (in_tail) { tail_acc = acc; in_tail = false; }
@@ -638,10 +681,10 @@ gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
     }
     // The launcher gives every wave at least `groups` pairs, so a tile is shared by two waves at most: the head
     // goes through LDS to the wave that holds the tail, which adds the two in this order and stores.
-    if (total > 0 && cg != 0) heads[wave * 64 + lane] = acc;
+    if (total > 0 && cg != 0) reinterpret_cast<v4f*>(line_buf)[lane] = acc;
     __syncthreads();
     if (has_tail) {
-        const v4f h = heads[(wave - 1) * 64 + lane];
+        const v4f h = reinterpret_cast<const v4f*>(line_buf - kWaveBuf)[lane];     // (the wave before this one)
         store(tail_tile, h + tail_acc);
     }
 }
@@ -657,17 +700,19 @@ static bool launch_gemm_wide(const void* A, const void* W, void* C, int M, int N
     const int steps = (K + 31) / 32, groups = (steps + kWideDepth - 1) / kWideDepth;
     const int a_stride = groups * kWideDepth * 32 + 16;
     const size_t rows_bytes = (size_t)M * a_stride * 2;
-    auto lds_of = [&](int wv) { return rows_bytes + (4 * wv * 16 + 16) * sizeof(float) + (size_t)wv * 64 * 16; };
+    const bool lines = g_lines_enabled && K >= 2048 && K % 64 == 0 && ldw % 64 == 0 && ((uintptr_t)W & 127) == 0;
+    auto lds_of = [&](int wv) { return rows_bytes + (4 * wv * 16 + 16) * sizeof(float) + (size_t)wv * (lines ? 16 * kLineRowBytes : 64 * 16); };
     // two blocks of 8 waves a compute unit; with many or long token rows one block of 16 waves, or of 8 when only that fits
     const bool two = 2 * lds_of(8) <= (size_t)kWideLdsLimit;
     const int wv = (two || lds_of(16) > (size_t)kWideLdsLimit) ? 8 : 16;
     const size_t lds = lds_of(wv);
     if (M > 16 || K < 8 || K % 8 || lds > (size_t)kWideLdsLimit) return false;
-    static bool raised[2][2][64] = {};                       // per kernel and device: it may use more than 64 KB of LDS
+    static bool raised[2][2][2][64] = {};                    // per kernel and device: it may use more than 64 KB of LDS
     int dev = 0;
     if (hipGetDevice(&dev) != hipSuccess || dev < 0 || dev >= 64) return false;
-    bool& done = raised[sizeof(TC) == 2 ? 1 : 0][wv == 8 ? 1 : 0][dev];
-    const void* fn = wv == 8 ? (const void*)gemm_wide_kernel<TC, 8> : (const void*)gemm_wide_kernel<TC, 16>;
+    bool& done = raised[sizeof(TC) == 2 ? 1 : 0][wv == 8 ? 1 : 0][lines ? 1 : 0][dev];
+    const void* fn = wv == 8 ? (lines ? (const void*)gemm_wide_kernel<TC, 8, true> : (const void*)gemm_wide_kernel<TC, 8, false>)
+                             : (lines ? (const void*)gemm_wide_kernel<TC, 16, true> : (const void*)gemm_wide_kernel<TC, 16, false>);
     if (!done) {
         if (hipFuncSetAttribute(fn, hipFuncAttributeMaxDynamicSharedMemorySize, kWideLdsLimit) != hipSuccess) {
             (void)hipGetLastError();
@@ -680,12 +725,12 @@ static bool launch_gemm_wide(const void* A, const void* W, void* C, int M, int N
     int blocks = cus * (two ? 2 : 1);
     if (blocks > tiles / wv) blocks = tiles / wv;
     if (blocks < 1) return false;
-    if (wv == 8)
-        hipLaunchKernelGGL((gemm_wide_kernel<TC, 8>), dim3(blocks), dim3(512), lds, stream, (const uint16_t*)A,
-                           (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, nf, a_stride);
-    else
-        hipLaunchKernelGGL((gemm_wide_kernel<TC, 16>), dim3(blocks), dim3(1024), lds, stream, (const uint16_t*)A,
-                           (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, nf, a_stride);
+#define IC_WIDE(WV, LN)                                                                                                   \
+    hipLaunchKernelGGL((gemm_wide_kernel<TC, WV, LN>), dim3(blocks), dim3(WV * 64), lds, stream, (const uint16_t*)A, \
+                       (const uint16_t*)W, (TC*)C, M, N, K, lda, ldw, ldc, alpha, nf, a_stride)
+    if (wv == 8) { if (lines) IC_WIDE(8, true); else IC_WIDE(8, false); }
+    else { if (lines) IC_WIDE(16, true); else IC_WIDE(16, false); }
+#undef IC_WIDE
     return true;
 }
 

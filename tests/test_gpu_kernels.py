@@ -630,6 +630,31 @@ def test_norm_split_over_two_products(M, N, K, N2):
         _close(act, P.plain_swiglu(gu[:, :N2 // 2], gu[:, N2 // 2:]), torch.bfloat16, factor=2)
 
 
+@pytest.mark.parametrize("out_dtype", [torch.float32, torch.bfloat16])
+@pytest.mark.parametrize("M,N,K", [(1, 33001, 2048), (7, 40000, 2112), (16, 32771, 2304)])
+def test_the_head_product_with_whole_line_weight_loads(M, N, K, out_dtype):
+    """Very many weight rows (the output head): from rows of 4 KB that are whole cache lines the kernel whose waves own
+    whole weight tiles reads them line by line through LDS; switched off it loads in operand layout.  The two add the same
+    products in the same order, so they agree to the bit, and both give the plain product."""
+    from infinicore_infer_amd.kernels.lib import get_lib
+    ops, lib = _ops(), get_lib()
+    g = torch.Generator().manual_seed(67)
+    a = torch.randn(M, K, generator=g).to(torch.bfloat16)
+    w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16)
+    ad, wd = a.to(DEV), w.to(DEV)
+    got = {}
+    try:
+        for on in (1, 0):
+            lib.ic_gemm_nt_lines_enable(on)
+            out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+            ops.gemm_nt(ad, wd, out, 0.25)
+            got[on] = out.cpu()
+    finally:
+        lib.ic_gemm_nt_lines_enable(1)
+    assert torch.equal(got[1], got[0])
+    _close(got[1], 0.25 * P.plain_linear(a, w), out_dtype, factor=20 if out_dtype == torch.float32 else 2)
+
+
 @pytest.mark.parametrize("M", [1, 3, 8, 16])
 @pytest.mark.parametrize("N,K", [(331, 192), (2304, 2304), (1000, 1536), (512, 8192 + 64), (12000, 640)])
 def test_whole_line_weight_loads_equal_loads_in_operand_layout(M, N, K):
