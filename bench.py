@@ -100,27 +100,31 @@ def time_prefill(engine, tokens, reps=6):
 
 def time_decode_scheduled(engine, batch, steps, warmup, vocab, seed=0):
     """``batch`` requests of PROMPT tokens go through the scheduler; once all of them decode, ``warmup``
-    untimed and ``steps`` timed scheduler steps (each: one token for every request)."""
+    untimed and ``steps`` timed steps (each: one token for every request)."""
     from infinicore_infer_amd.engine.scheduler import Scheduler
     from infinicore_infer_amd.engine.tasks import InferTask
     g = torch.Generator().manual_seed(seed)
-    sch = Scheduler(engine, max_batch_tokens=max(PROMPT, batch), chunk_size=PROMPT)
+    sch = Scheduler(engine, max_batch_tokens=max(PROMPT, batch), chunk_size=PROMPT, overlap=True)
     for i in range(batch):
         toks = torch.randint(0, vocab, (PROMPT,), generator=g).tolist()
         sch.add(InferTask("d%d" % i, toks, 1 << 30, temperature=0.0, topk=1, end_tokens=[],
                           max_new_tokens=warmup + steps + batch + 8))     # the first ones decode while the others' prompts run
     while sch.waiting or any(not r.decoding for r in sch.running):
         sch.step()
-    for _ in range(warmup):
-        assert len(sch.step()) == batch
+    # (decoding runs one step ahead of the host: a call issues at most one step and returns the tokens of the one before)
+    first = sch.n_steps
+    while sch.n_steps < first + warmup:
+        sch.step()
     _sync()
     ctx0 = engine.length("d0")
+    first = sch.n_steps
     t0 = time.perf_counter()
-    for _ in range(steps):
+    while sch.n_steps < first + steps:
         sch.step()
     _sync()
     dt = time.perf_counter() - t0
     ctx1 = engine.length("d0")
+    assert sch.n_steps == first + steps and ctx1 - ctx0 == steps
     assert len(sch.running) == batch and sch.n_preempted == 0
     for i in range(batch):
         sch.abort("d%d" % i)

@@ -140,6 +140,9 @@ class Engine:
         self._graph_ws: Optional[Workspace] = None      # shared by all recorded steps of a natively stepped model
         self.graph_steps = 0         # steps that took the recorded path (the recording one included)
         self.graph_replays = 0       # of these, replays of an existing recording
+        self.steps_ahead = 0         # recorded steps that took their tokens from the device (step_ahead)
+        self._ahead_out = None       # two sets of buffers for tokens sampled without waiting, used in turn
+        self._ahead_turn = 0
         self.graphs_evicted = 0
         self.graph_after = max(1, int(graph_after))
         self._graph_seen: "OrderedDict[tuple, int]" = OrderedDict()     # shapes not yet recorded: how often they came
@@ -284,6 +287,40 @@ class Engine:
         for e in entries:
             self.cache.trim(e.req_id)
         self.steps_run += 1
+        return logits
+
+    def step_ahead(self, entries: Sequence[StepEntry], device_tokens):
+        """The next decode step of requests whose last tokens the host has not seen yet: every entry is one admitted
+        request's single next token with its logits wanted, its ``tokens`` a placeholder ([0]); the tokens themselves
+        are ``device_tokens`` (int32 [len(entries)] on the device, what ``sample_ahead`` returned for the step before,
+        in the order of the entries).  Only a recorded step can run so: returns its logits, or None with nothing
+        changed when there is no recording for this batch size and context yet, when pages are missing or anything
+        else is amiss (the caller then waits for the tokens and calls ``step``)."""
+        R = len(entries)
+        if (not self.use_graphs or R == 0 or R > self.graph_max_batch or self._has_window
+                or device_tokens is None or device_tokens.numel() != R or device_tokens.dtype != torch.int32):
+            return None
+        reqs = self.cache.requests
+        longest = 0
+        for e in entries:
+            req = reqs.get(e.req_id)
+            if req is None:
+                return None
+            longest = max(longest, req.length)
+        g = self._graphs.get((R, _context_bucket(longest + 1)))
+        if g is None or g.graph is None:
+            return None
+        starts = self._append_single_tokens(entries)
+        if starts is None:
+            return None
+        try:
+            logits = self._graph_step(entries, starts, device_tokens)
+        except BaseException:
+            for e, p0 in zip(entries, starts):
+                self.cache.truncate(e.req_id, p0)
+            raise
+        self.steps_run += 1
+        self.steps_ahead += 1
         return logits
 
     def _append_single_tokens(self, entries):
@@ -461,7 +498,7 @@ class Engine:
         return ctx
 
     # ---- decode steps as captured graphs ------------------------------------------------------------
-    def _graph_step(self, entries, starts):
+    def _graph_step(self, entries, starts, device_tokens=None):
         """A step of single tokens, one per request, all logits wanted.  The kernels of
         such a step differ from step to step only in the integers they read (tokens,
         positions, slots, block tables), so the launch sequence is captured once per
@@ -495,6 +532,8 @@ class Engine:
         g.fill(self, entries, starts)
         g.meta.copy_(g.host, non_blocking=True)
         g.copied.record()
+        if device_tokens is not None:               # (only with a recording at hand: step_ahead has looked)
+            g.ctx.tokens.copy_(device_tokens)
         g.ctx.max_position = max(starts)
         g.ctx.req_pos = list(starts)
         g.ctx.req_ids = [e.req_id for e in entries]
@@ -569,6 +608,44 @@ class Engine:
             k = torch.tensor(list(top_k), dtype=torch.int32).to(self.device)
             ops.sample(logits, out, f[0].contiguous(), k, f[1].contiguous(), f[2].contiguous())
         return out.cpu().tolist()
+
+    def sample_ahead(self, logits, temperature=None, top_k=None, top_p=None, uniform=None):
+        """As ``sample``, without waiting for the device: returns (the tokens on the device, int32 [rows], and a
+        function that waits for them and returns them as a list).  The device tokens can go straight into
+        ``step_ahead``; two sets of buffers are used in turn, so a result stays readable until the call after next."""
+        R = logits.shape[0]
+        if self._ahead_out is None:
+            n = max(self.graph_max_batch, 1)
+            self._ahead_out = [dict(tokens=torch.empty(n, dtype=torch.int32, device=self.device),
+                                    host=torch.empty(n, dtype=torch.int32, pin_memory=True), done=torch.cuda.Event(),
+                                    f=torch.empty(3, n, dtype=torch.float32, device=self.device),
+                                    f_host=torch.empty(3, n, dtype=torch.float32, pin_memory=True),
+                                    k=torch.empty(n, dtype=torch.int32, device=self.device),
+                                    k_host=torch.empty(n, dtype=torch.int32, pin_memory=True)) for _ in range(2)]
+            for b in self._ahead_out:
+                b["done"].record()
+        if R > self._ahead_out[0]["tokens"].numel():
+            raise ValueError("sample_ahead takes at most %d rows" % self._ahead_out[0]["tokens"].numel())
+        self._ahead_turn ^= 1
+        b = self._ahead_out[self._ahead_turn]
+        b["done"].synchronize()                     # what this set of buffers held two calls ago has been copied out
+        out, host, done = b["tokens"][:R], b["host"], b["done"]
+        if temperature is None:
+            ops.argmax(logits, out, self.ws.buffer("argmax_val", (64 * R,), torch.float32),
+                       self.ws.buffer("argmax_idx", (64 * R,), torch.int32))
+        else:
+            b["f_host"][:, :R] = torch.tensor([list(temperature), list(top_p), list(uniform)], dtype=torch.float32)
+            b["k_host"][:R] = torch.tensor(list(top_k), dtype=torch.int32)
+            b["f"].copy_(b["f_host"], non_blocking=True)        # (pinned: the host does not wait for the device)
+            b["k"].copy_(b["k_host"], non_blocking=True)
+            ops.sample(logits, out, b["f"][0, :R], b["k"][:R], b["f"][1, :R], b["f"][2, :R])
+        host[:R].copy_(out, non_blocking=True)
+        done.record()
+
+        def wait() -> List[int]:
+            done.synchronize()
+            return host[:R].tolist()
+        return out, wait
 
 
 class _DecodeGraph:

@@ -23,7 +23,15 @@ there is no token budget and memory is committed per whole-context slab
     the FRONT of the waiting queue with prompt + generated tokens to be
     recomputed; its random draws depend only on (seed, id, token index), so the
     continuation is the same.  A request that cannot fit even alone finishes
-    with finish_reason "length".
+    with finish_reason "length";
+  * with ``overlap`` (and an engine that has ``step_ahead`` and ``sample_ahead``) pure decoding runs one step
+    ahead of the host: while the device computes a step, the host issues the next one, whose input tokens
+    the device takes from its own sampler's output, and only then reads the tokens of the step before.  The
+    device then never waits for the host's bookkeeping.  ``step`` returns a step's tokens one call later; what
+    cannot be known without the tokens (an end token) is found a step late: that request's extra token is dropped
+    and its pages are given back then.  Whenever something else is due (a waiting request, a request that ends
+    by length, missing pages, a batch the engine has no recording for) the host waits for the tokens and the
+    step after is planned as without overlap.  The tokens are the same with and without.
 
 The scheduler only needs ``engine.cache`` (a CacheManager), ``engine.step``,
 ``engine.sample``, ``engine.add_request`` and ``engine.free``, so its decisions
@@ -37,6 +45,15 @@ from ..cache import OutOfPages
 from ..sampling import uniform_draw
 from .engine import StepEntry
 from .tasks import InferTask
+
+
+@dataclass
+class _Ahead:
+    """A step whose sampled tokens the host has not read yet."""
+    rows: list                       # the requests whose tokens it samples, in the rows' order
+    pos: List[int]                   # each request's cache length after the step
+    device_tokens: object            # the tokens on the device
+    wait: object                     # waits for them and returns them as a list
 
 
 @dataclass(eq=False)               # compared by identity: membership tests must not compare token lists
@@ -53,7 +70,7 @@ class _Running:
 
 class Scheduler:
     def __init__(self, engine, max_batch_tokens: int = 2048, chunk_size: int = 512,
-                 max_running: Optional[int] = None, prefix_cache: bool = False):
+                 max_running: Optional[int] = None, prefix_cache: bool = False, overlap: bool = False):
         if max_batch_tokens < 1 or chunk_size < 1:
             raise ValueError("max_batch_tokens and chunk_size must be positive")
         self.engine = engine
@@ -72,6 +89,11 @@ class Scheduler:
         # pages back) and no fixed-size state exists (a state cannot be cut back to a prefix).
         self.prefix_cache = (bool(prefix_cache) and all(g.kind == "full" for g in self.cache.groups)
                              and not getattr(engine, "has_state", False))
+        # decoding one step ahead of the host: not together with kept caches (a cache would be kept with a token more)
+        self.overlap = (bool(overlap) and not self.prefix_cache and hasattr(engine, "step_ahead")
+                        and hasattr(engine, "sample_ahead"))
+        self._ahead: Optional[_Ahead] = None
+        self.n_ahead = 0                 # steps issued before the tokens of the step before were read
         self.idle: "OrderedDict[object, List[int]]" = OrderedDict()    # kept cache id -> the tokens it holds, oldest first
         self._idle_serial = 0
         self.n_prefix_hits = 0
@@ -84,7 +106,7 @@ class Scheduler:
         self.waiting.append(_Running(task, list(task.prompt)))
 
     def has_unfinished(self) -> bool:
-        return bool(self.waiting or self.running)
+        return bool(self.waiting or self.running or self._ahead is not None)
 
     def abort(self, task_id) -> None:
         for r in list(self.running):
@@ -276,8 +298,69 @@ class Scheduler:
             return self.plan()
         return plan
 
+    # ---- one step ahead of the host ---------------------------------------------------------------------
+    def _sampling_arguments(self, rows, ahead: int):
+        """() for greedy rows, else the per-row lists ``engine.sample`` takes; ``ahead``: tokens of each row that are
+        sampled but not yet in ``generated`` (the random draw is a function of the token's index)."""
+        tasks = [r.task for r in rows]
+        if all(t.temperature == 0 or t.topk == 1 for t in tasks):
+            return ()
+        return ([t.temperature for t in tasks], [t.topk for t in tasks], [t.topp for t in tasks],
+                [uniform_draw(t.seed, t.id, len(t.generated) + ahead) for t in tasks])
+
+    def _ends_by_length(self, t: InferTask, pos: int, n_generated: int) -> bool:
+        return (pos >= t.max_tokens or (self.cache.max_positions is not None and pos >= self.cache.max_positions)
+                or (t.max_new_tokens is not None and n_generated >= t.max_new_tokens))
+
+    def _take(self, rows, tokens, positions) -> List[Tuple[InferTask, int]]:
+        """Book the tokens a step sampled: append, report, finish.  Rows of requests that have ended meanwhile
+        (an end token found a step late, a cancellation) are dropped."""
+        out: List[Tuple[InferTask, int]] = []
+        for r, tok, pos in zip(rows, tokens, positions):
+            t = r.task
+            if t.finish_reason is not None:
+                continue
+            t.generated.append(int(tok))
+            t.pos = pos
+            out.append((t, int(tok)))
+            if tok in t.end_tokens:
+                self._finish(r, "stop")
+            elif self._ends_by_length(t, pos, len(t.generated)):
+                self._finish(r, "length")           # the task's own limit, or the model has no position left
+        return out
+
+    def _issue_ahead(self, prev: _Ahead) -> Optional[_Ahead]:
+        """The step after ``prev`` from the device's own tokens, when it is plain decoding of the same requests
+        and nothing else is due; None when the host has to see the tokens first."""
+        if self.waiting or len(self.running) != len(prev.rows) or len(prev.rows) > self.max_batch_tokens:
+            return None
+        for r, mine, pos in zip(prev.rows, self.running, prev.pos):
+            t = r.task
+            if r is not mine or t.finish_reason is not None or self._ends_by_length(t, pos, len(t.generated) + 1):
+                return None
+        entries = [StepEntry(r.task.id, [0], [0]) for r in prev.rows]
+        first = [self.cache.length(r.task.id) for r in prev.rows]
+        logits = self.engine.step_ahead(entries, prev.device_tokens)
+        if logits is None:
+            return None
+        self.last_plan = [(r.task.id, p, 1) for r, p in zip(prev.rows, first)]
+        self.n_steps += 1
+        self.n_ahead += 1
+        dev, wait = self.engine.sample_ahead(logits, *self._sampling_arguments(prev.rows, 1))
+        return _Ahead(prev.rows, [p + 1 for p in first], dev, wait)
+
+    def _step_behind(self) -> List[Tuple[InferTask, int]]:
+        """A step is on the device whose tokens the host has not read: issue the one after it if that can be done
+        without them, then read and book them."""
+        prev = self._ahead
+        self._ahead = self._issue_ahead(prev)
+        return self._take(prev.rows, prev.wait(), prev.pos)
+
     def step(self) -> List[Tuple[InferTask, int]]:
-        """Run one step; returns (task, new token) for every request that got a token."""
+        """Run one step; returns (task, new token) for every request that got a token (with ``overlap``, while
+        decoding runs ahead of the host: the tokens of the step before the one this call issued)."""
+        if self._ahead is not None:
+            return self._step_behind()
         plan = self.plan()
         if not plan:
             return []
@@ -295,28 +378,18 @@ class Scheduler:
             if not r.decoding:
                 r.cursor += n
         self.n_steps += 1
-        out: List[Tuple[InferTask, int]] = []
-        if samplers:
-            tasks = [r.task for r in samplers]
-            if all(t.temperature == 0 or t.topk == 1 for t in tasks):
-                tokens = self.engine.sample(logits)
-            else:
-                tokens = self.engine.sample(
-                    logits, [t.temperature for t in tasks], [t.topk for t in tasks], [t.topp for t in tasks],
-                    [uniform_draw(t.seed, t.id, len(t.generated)) for t in tasks])
-            for r, tok in zip(samplers, tokens):
-                t = r.task
-                t.generated.append(int(tok))
-                t.pos = self.cache.length(t.id)
-                out.append((t, int(tok)))
-                if tok in t.end_tokens:
-                    self._finish(r, "stop")
-                elif t.pos >= t.max_tokens or (self.cache.max_positions is not None
-                                               and t.pos >= self.cache.max_positions):
-                    self._finish(r, "length")       # the task's own limit, or the model has no position left
-                elif t.max_new_tokens is not None and len(t.generated) >= t.max_new_tokens:
-                    self._finish(r, "length")
-        return out
+        if not samplers:
+            return []
+        positions = [self.cache.length(r.task.id) for r in samplers]
+        if (self.overlap and not self.waiting and len(samplers) == len(self.running)
+                and all(r.decoding for r in self.running)):
+            # every running request decodes from here on: do not wait for this step's tokens, the next call
+            # issues the step after it first
+            dev, wait = self.engine.sample_ahead(logits, *self._sampling_arguments(samplers, 0))
+            self._ahead = _Ahead(list(samplers), positions, dev, wait)
+            return []
+        tokens = self.engine.sample(logits, *self._sampling_arguments(samplers, 0))
+        return self._take(samplers, tokens, positions)
 
     def run(self, on_step=None) -> List[InferTask]:
         """Step until every request has finished.  ``on_step(new, seconds)``, when given, is called

@@ -159,7 +159,7 @@ class MiniCPMForCausalLM:
             sched = self._scheduler
             sched.max_batch_tokens, sched.chunk_size = max_batch_tokens, chunk_size
         else:
-            sched = Scheduler(self.engine, max_batch_tokens=max_batch_tokens, chunk_size=chunk_size)
+            sched = Scheduler(self.engine, max_batch_tokens=max_batch_tokens, chunk_size=chunk_size, overlap=True)
         tasks = [InferTask("g%d" % i, list(p), self.max_context_len(), temperature_, topk_, topp_,
                            self.eos_token_id, seed=seed, max_new_tokens=max_new_tokens)
                  for i, p in enumerate(prompts)]

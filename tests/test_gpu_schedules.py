@@ -269,6 +269,50 @@ def test_preemption_under_temperature_sampling_gives_the_same_tokens(tmp_path_fa
         assert sum(common) >= 40 and max(common) >= 20
 
 
+# ---- decoding one step ahead of the host --------------------------------------------------------------------------------
+@pytest.mark.parametrize("native", [True, False])
+@pytest.mark.parametrize("temperature", [0.0, 0.8])
+def test_decoding_ahead_of_the_host_on_the_engine(tmp_path_factory, temperature, native):
+    """``overlap``: recorded decode steps take their input tokens from the sampler's output on the device while the
+    host still books the step before.  Six requests of different lengths, one of which ends on an end token (chosen
+    from the run without overlap), greedy and with temperature sampling, float32 so that both runs see the same
+    logits: the same tokens and finish reasons as without overlap, most decode steps issued ahead, every page back."""
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.engine.scheduler import Scheduler
+    from infinicore_infer_amd.engine.tasks import InferTask
+    cfg = H.CONFIGS["A"][0]
+    folder = H.make_model_dir(tmp_path_factory.getbasetemp(), "A")
+    prompts = [H.random_tokens(cfg["vocab_size"], n, 300 + i) for i, n in enumerate([9, 30, 17, 5, 22, 12])]
+    news = [40, 25, 33, 40, 12, 40]
+
+    def run(overlap, end_tokens):
+        eng = Engine.from_dir(folder, dtype=torch.float32, max_tokens=6 * 96, page_size=16, max_requests=6, use_native=native)
+        sch = Scheduler(eng, max_batch_tokens=64, chunk_size=32, overlap=overlap)
+        assert sch.overlap == overlap
+        tasks = [InferTask("t%d" % i, p, 256, temperature=temperature, topk=1 if temperature == 0 else 30, topp=0.9,
+                           end_tokens=end_tokens, seed=11, max_new_tokens=n) for i, (p, n) in enumerate(zip(prompts, news))]
+        for t in tasks[:4]:
+            sch.add(t)
+        calls = 0
+        while sch.has_unfinished() or calls < 12:
+            if calls == 11:                       # two more arrive while the others decode ahead
+                sch.add(tasks[4]); sch.add(tasks[5])
+            sch.step()
+            calls += 1
+        eng.cache.check_invariants()
+        assert eng.cache.free_pages(0) == eng.cache.pools[0].num_pages and sch.n_preempted == 0
+        return [(t.generated, t.finish_reason) for t in tasks], sch, eng
+
+    base, _, _ = run(False, [])
+    stop = base[0][0][20]                          # the first request will end here
+    want, s0, e0 = run(False, [stop])
+    got, s1, e1 = run(True, [stop])
+    assert got == want
+    assert want[0][1] == "stop" and len(want[0][0]) <= 21 and any(r == "length" for _, r in want)
+    assert s0.n_ahead == 0 and e0.steps_ahead == 0
+    assert s1.n_ahead == e1.steps_ahead and s1.n_ahead >= 20
+
+
 # ---- the command line ---------------------------------------------------------------------------------------------------
 @pytest.mark.parametrize("dname", ["float32", "bfloat16"])
 @pytest.mark.parametrize("name", ["A", "B"])

@@ -299,3 +299,95 @@ def test_prefix_cache_stays_off_where_keys_are_given_back():
     eng.cache = CacheManager([GroupSpec("window", 1, 16, 32, (0,))], 8, 16, 4, None)
     assert not Scheduler(eng, prefix_cache=True).prefix_cache
     assert Scheduler(FakeEngine(num_pages=8), prefix_cache=True).prefix_cache
+
+
+# ---- decoding one step ahead of the host ------------------------------------------------------------------------------
+class AheadEngine(FakeEngine):
+    """The stand-in engine with the two calls that decoding ahead needs.  Its 'device tokens' are a function that
+    yields the tokens, so that a test can see that the scheduler never looked at them before the next step was
+    issued.  ``refuse`` makes step_ahead give up now and then, as a real engine does for a batch it has no
+    recording of."""
+
+    def __init__(self, *args, refuse=0, **kw):
+        super().__init__(*args, **kw)
+        self.refuse, self.ahead_calls, self.ahead_steps, self.reads = refuse, 0, 0, []
+
+    def step_ahead(self, entries, device_tokens):
+        from infinicore_infer_amd.engine import StepEntry
+        self.ahead_calls += 1
+        if self.refuse and self.ahead_calls % self.refuse == 0:
+            return None
+        if sum(self.cache.pages_needed(e.req_id, 1)[0] for e in entries) > self.cache.free_pages(0):
+            return None
+        assert all(e.tokens == [0] and list(e.want) == [0] for e in entries)
+        self.ahead_steps += 1
+        self.reads.append("issue")
+        return self.step([StepEntry(e.req_id, [t], [0]) for e, t in zip(entries, device_tokens())])
+
+    def sample_ahead(self, logits, temperature=None, top_k=None, top_p=None, uniform=None):
+        rows = list(logits)
+
+        def wait():
+            self.reads.append("read")
+            return rows
+        return (lambda: rows), wait
+
+
+def _run_requests(overlap, num_pages, refuse, arrivals, end=()):
+    eng = AheadEngine(num_pages, page_size=16, max_requests=4, refuse=refuse) if overlap else FakeEngine(num_pages, max_requests=4)
+    s = Scheduler(eng, max_batch_tokens=40, chunk_size=24, overlap=overlap)
+    tasks, calls = [], 0
+    pending = sorted(arrivals, key=lambda a: a[0])
+    while pending or s.has_unfinished():
+        while pending and pending[0][0] <= calls:
+            _, name, prompt, new = pending.pop(0)
+            tasks.append(_task(name, prompt, new, end))
+            s.add(tasks[-1])
+        s.step()
+        calls += 1
+        assert calls < 5000
+    eng.cache.check_invariants()
+    assert eng.cache.free_pages(0) == num_pages and not eng.history
+    return {t.id: (t.generated, t.finish_reason) for t in tasks}, s, eng
+
+
+@pytest.mark.parametrize("refuse", [0, 3])
+@pytest.mark.parametrize("num_pages", [64, 6])
+@pytest.mark.parametrize("seed", [5, 7])
+def test_decoding_ahead_of_the_host_gives_the_same_tokens(seed, num_pages, refuse):
+    """With ``overlap`` the scheduler issues a decode step before it has read the tokens of the step before.  Requests
+    that arrive while others decode, end tokens (found a step late: the extra token is dropped), different lengths,
+    few pages (preemption) and an engine that refuses now and then: tokens and finish reasons are those of the run
+    without overlap, and every page comes back."""
+    import random
+    rng = random.Random(seed)
+    arrivals = [(at, "r%d" % i, [rng.randrange(VOCAB) for _ in range(rng.randint(3, 40))], rng.randint(1, 40))
+                for i, at in enumerate([0, 0, 0, 0, 5, 9, 30, 31, 60])]
+    end = (7,)
+    want, s0, _ = _run_requests(False, num_pages, 0, arrivals, end)
+    got, s1, eng = _run_requests(True, num_pages, refuse, arrivals, end)
+    assert got == want
+    assert any(reason == "stop" for _, reason in want.values()) and any(reason == "length" for _, reason in want.values())
+    assert eng.ahead_steps == s1.n_ahead > 0
+    if num_pages == 64:
+        assert s1.n_ahead >= 15 and s0.n_preempted == s1.n_preempted == 0
+    else:
+        assert s0.n_preempted > 0 and s1.n_preempted > 0
+
+
+def test_decoding_ahead_issues_the_next_step_before_it_reads_the_tokens():
+    eng = AheadEngine(64, max_requests=4)
+    s = Scheduler(eng, max_batch_tokens=64, chunk_size=64, overlap=True)
+    for i in range(3):
+        s.add(_task("q%d" % i, [1 + i, 2, 3], 12))
+    assert len(s.step()) == 0 and eng.reads == []               # the prompts' step: its tokens are not waited for
+    for k in range(5):
+        out = s.step()
+        assert len(out) == 3 and eng.reads[-2:] == ["issue", "read"]      # the step after is on its way first
+    assert s.n_ahead == 5 and s.n_steps == 6
+    done = s.run()
+    assert sorted(len(t.generated) for t in done) == [12, 12, 12]
+    assert [t.generated for t in sorted(done, key=lambda t: t.id)] == [_expected([1 + i, 2, 3], 12) for i in range(3)]
+    # without the two calls, or with kept caches, the scheduler stays as it was
+    assert not Scheduler(FakeEngine(8), overlap=True).overlap
+    assert not Scheduler(AheadEngine(8), overlap=True, prefix_cache=True).overlap
