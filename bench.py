@@ -181,16 +181,20 @@ def run_mixed(args):
     prompts = [torch.randint(0, conf.vocab_size, (l,), generator=g).tolist() for l in lens]
 
     def run():
-        sch = Scheduler(engine, max_batch_tokens=budget, chunk_size=chunk)
+        sch = Scheduler(engine, max_batch_tokens=budget, chunk_size=chunk, overlap=True)
         for i, toks in enumerate(prompts):
             sch.add(InferTask(i, toks, conf.max_position_embeddings, temperature=0.0, topk=1, end_tokens=[], max_new_tokens=gen))
         _sync()
         t0 = time.perf_counter()
         steps = []
         while sch.has_unfinished():
-            s0 = time.perf_counter()
+            s0, issued = time.perf_counter(), sch.n_steps
             sch.step()
-            steps.append((time.perf_counter() - s0, sum(n for _, _, n in sch.last_plan)))
+            took = time.perf_counter() - s0
+            if sch.n_steps > issued:                    # the call issued a step (while decoding runs ahead it also waited for the one before)
+                steps.append((took, sum(n for _, _, n in sch.last_plan)))
+            elif steps:                                 # it only read the tokens of the step in flight
+                steps[-1] = (steps[-1][0] + took, steps[-1][1])
         _sync()
         return time.perf_counter() - t0, steps, sch.n_preempted
 
