@@ -91,7 +91,7 @@ class Scheduler:
                              and not getattr(engine, "has_state", False))
         # decoding one step ahead of the host: not together with kept caches (a cache would be kept with a token more)
         self.overlap = (bool(overlap) and not self.prefix_cache and hasattr(engine, "step_ahead")
-                        and hasattr(engine, "sample_ahead"))
+                        and hasattr(engine, "sample_ahead") and getattr(engine, "use_graphs", True))
         self._ahead: Optional[_Ahead] = None
         self.n_ahead = 0                 # steps issued before the tokens of the step before were read
         self.idle: "OrderedDict[object, List[int]]" = OrderedDict()    # kept cache id -> the tokens it holds, oldest first
