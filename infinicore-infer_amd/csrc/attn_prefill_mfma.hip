@@ -33,11 +33,9 @@
 // Cache layout of one layer: K and V planes [num_pages, n_kv_heads, page_size, head_dim].
 #include "common.h"
 
-// Arrival counters of the split walk, one per (tile, head): zero when the library is loaded, and put back to zero
-// by the block that merges.  Launches that split and overlap in time on one device would share them: the engine
-// issues a step's kernels on one stream.
+// Arrival counters of the split walk, one per (tile, head), in memory of the caller's: zero before the first launch,
+// and put back to zero by the block that merges, so launches that follow each other on a stream share one buffer.
 constexpr int kPfCounters = 1 << 16;
-__device__ int g_pf_arrivals[kPfCounters];
 
 typedef __bf16 bf16x8 __attribute__((ext_vector_type(8)));
 typedef float v16f __attribute__((ext_vector_type(16)));
@@ -62,7 +60,7 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                          const uint16_t* __restrict__ kcache, const uint16_t* __restrict__ vcache,
                          const int* __restrict__ block_tables, int bt_stride, const int4* __restrict__ tiles,
                          int n_tiles, int nh, int nkvh, int page_shift, float scale_log2e, int window,
-                         int parts, int part_len, float* __restrict__ scratch) {
+                         int parts, int part_len, float* __restrict__ scratch, int* __restrict__ counters) {
     constexpr int NC = DH / 16;           // 16-wide chunks of the head dimension
     constexpr int ND = DH / 32;           // 32-row tiles of O^T
     constexpr int KS = DH + kPfPad;       // row stride of Ks (elements): 16-byte reads of 8 consecutive rows cover all banks
@@ -359,10 +357,10 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         // for stores to memory (waves of a block share their unit's cache, so a barrier need not)
         asm volatile("s_waitcnt vmcnt(0)" ::: "memory");
         __syncthreads();
-        if (tid == 0) arrived = atomicAdd(&g_pf_arrivals[slot], 1);
+        if (tid == 0) arrived = atomicAdd(&counters[slot], 1);
         __syncthreads();
         if (arrived != n_parts - 1) return;
-        if (tid == 0) g_pf_arrivals[slot] = 0;               // for the next launch
+        if (tid == 0) counters[slot] = 0;                    // for the next launch
         for (int p = 0; p < n_parts; ++p) {
             if (p == part) continue;
             const float* other = scratch + ((size_t)slot * parts + p) * PF;
@@ -399,6 +397,7 @@ IC_EXPORT int ic_attn_prefill_supported(int dtype, int dh, int page_size) {
 }
 
 IC_EXPORT int ic_attn_prefill_tile_rows() { return kPfRows; }
+IC_EXPORT int ic_attn_prefill_counter_ints() { return kPfCounters; }
 
 // Floats of scratch memory that a walk cut into `parts` needs: every (tile, head, part) keeps a maximum, a sum and O^T per row.
 IC_EXPORT long long ic_attn_prefill_scratch_floats(int n_tiles, int nh, int dh, int parts) {
@@ -442,7 +441,7 @@ IC_EXPORT int ic_attn_prefill_split(const void* q, int q_stride, void* out, int 
                                     const void* kcache, const void* vcache, const int* block_tables,
                                     int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
                                     int page_size, float scale, int window, int groups, int parts, int part_len,
-                                    float* scratch, long long scratch_floats, hipStream_t stream) {
+                                    float* scratch, long long scratch_floats, int* counters, hipStream_t stream) {
     if (n_tiles <= 0) return IC_OK;
     if (!ic_attn_prefill_supported(dtype, dh, page_size)) return IC_ERR_UNSUPPORTED;
     int page_shift = 0;
@@ -452,7 +451,7 @@ IC_EXPORT int ic_attn_prefill_split(const void* q, int q_stride, void* out, int 
         ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15) || ((uintptr_t)tiles & 15)) return IC_ERR_ARG;
     if (parts < 1) parts = 1;
     if (parts > 1) {
-        if (groups == 2 || part_len < 1 || parts > 64 || (long long)nh * n_tiles > kPfCounters || !scratch ||
+        if (groups == 2 || part_len < 1 || parts > 64 || (long long)nh * n_tiles > kPfCounters || !scratch || !counters ||
             ((uintptr_t)scratch & 15) || scratch_floats < ic_attn_prefill_scratch_floats(n_tiles, nh, dh, parts) ||
             (long long)nh * n_tiles * parts > 0x7fffffffLL) return IC_ERR_ARG;
         groups = 1;
@@ -476,7 +475,7 @@ IC_EXPORT int ic_attn_prefill_split(const void* q, int q_stride, void* out, int 
     hipLaunchKernelGGL((attn_prefill_mfma_kernel<DD, ST, GG, PP>), grid, dim3(256 * GG), 0, stream, (const uint16_t*)q, \
                        q_stride, (uint16_t*)out, out_stride, (const uint16_t*)kcache, (const uint16_t*)vcache,      \
                        block_tables, bt_stride, (const int4*)tiles, n_tiles, nh, nkvh, page_shift, sl2, window,      \
-                       parts, part_len, scratch)
+                       parts, part_len, scratch, counters)
 #define IC_PF_GROUPS(DD, ST) do { if (two_groups) { if (page64) IC_PF_LAUNCH(DD, ST, 2, true); else IC_PF_LAUNCH(DD, ST, 2, false); } \
                                   else { if (page64) IC_PF_LAUNCH(DD, ST, 1, true); else IC_PF_LAUNCH(DD, ST, 1, false); } } while (0)
     if (dh == 64) { if (staged) IC_PF_GROUPS(64, true); else IC_PF_GROUPS(64, false); }
@@ -493,7 +492,7 @@ IC_EXPORT int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int
                                      int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
                                      int page_size, float scale, int window, int groups, hipStream_t stream) {
     return ic_attn_prefill_split(q, q_stride, out, out_stride, dtype, kcache, vcache, block_tables, bt_stride, tiles,
-                                 n_tiles, nh, nkvh, dh, page_size, scale, window, groups, 1, 0, nullptr, 0, stream);
+                                 n_tiles, nh, nkvh, dh, page_size, scale, window, groups, 1, 0, nullptr, 0, nullptr, stream);
 }
 
 IC_EXPORT int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype,

@@ -17,6 +17,8 @@
 
 namespace {
 
+// The thresholds below are read by the ic_rule_* functions alone; the step function here and the parts' Python
+// forward both ask those functions, so a rule is written once.
 constexpr int kFewRows = 16;        // up to here the few-row products beat the library
 constexpr int kMidRows = 64;        // up to here the sliced product beats it for results as wide as the model
 constexpr int kMaxSumsqParts = 256; // column blocks of sums of squares a product takes as row factors
@@ -42,6 +44,52 @@ struct Deferred {
 };
 
 }  // namespace
+
+// ---- which kernel takes what: the one home of the dispatch rules ----------------------------------------------------------
+IC_EXPORT int ic_rule_few_rows() { return kFewRows; }
+IC_EXPORT int ic_rule_sumsq_parts_max() { return kMaxSumsqParts; }
+
+IC_EXPORT int ic_rule_own_product(int a_dtype, int w_dtype, int c_dtype, int rows) {
+    return rows <= kFewRows && a_dtype == IC_BF16 && ic_gemm_nt_supported(a_dtype, w_dtype, c_dtype);
+}
+
+IC_EXPORT int ic_rule_qkv_fused(int dtype, int rows, int K, int lda, int ldw, int head_dim, int rot_dim, int kv_heads_written,
+                                int row_factors_owed) {
+    if (dtype != IC_BF16 || kv_heads_written <= 0 || rot_dim != head_dim || !ic_gemm_qkv_rope_supported(IC_BF16, head_dim)) return 0;
+    if (rows <= kFewRows) return 1;
+    return !row_factors_owed && rows <= ic_gemm_nt_epilogue_rows(2, K, lda, ldw);
+}
+
+IC_EXPORT int ic_rule_gate_up_fused(int dtype, int rows, int K, int lda, int ldw, int row_factors_owed) {
+    if (dtype != IC_BF16) return 0;
+    if (rows <= kFewRows) return 1;
+    return !row_factors_owed && rows <= ic_gemm_nt_epilogue_rows(1, K, lda, ldw);
+}
+
+IC_EXPORT int ic_rule_tail(int dtype, int rows, int N, int K, int lda, int ldw) {
+    if (dtype != IC_BF16 || rows <= 0) return IC_TAIL_PLAIN;
+    if (rows <= kMidRows && N % 4 == 0 && ic_gemm_splitk_supported(rows, N, K, lda, ldw) && ic_gemm_splitk_pays(rows, N, K))
+        return IC_TAIL_SLICES;
+    if (rows <= kFewRows && ic_gemm_nt_residual_parts(N) <= kMaxSumsqParts) return IC_TAIL_SPLIT_NORM;
+    return IC_TAIL_PLAIN;
+}
+
+IC_EXPORT int ic_rule_attention(int dtype, int head_dim, int page_size, int n_decode_rows, int n_tiles) {
+    const bool dec_ok = ic_attn_decode_supported(dtype, head_dim) != 0;
+    const bool pre_ok = ic_attn_prefill_supported(dtype, head_dim, page_size) != 0;
+    const bool use_dec = dec_ok && n_decode_rows > 0 && (pre_ok || n_tiles == 0);
+    const bool use_pre = pre_ok && n_tiles > 0 && (dec_ok || n_decode_rows == 0);
+    if (!((use_dec || n_decode_rows == 0) && (use_pre || n_tiles == 0))) return IC_ATTN_GENERAL;
+    return (use_dec ? IC_ATTN_SINGLE_TOKENS : 0) | (use_pre ? IC_ATTN_PORTIONS : 0);
+}
+
+IC_EXPORT int ic_rule_context_bucket(int n_keys) {
+    int b = 256;
+    while (b < n_keys) b *= 2;
+    if (b <= 1024) return b;
+    const int q = b / 8;
+    return (n_keys + q - 1) / q * q;
+}
 
 struct IcDecoder {
     IcDecoderMeta meta;
@@ -75,6 +123,7 @@ struct IcDecoder {
 
     // into how many parts the walks of a step's prompt tiles are cut (1: not at all), and key tiles per part
     int tile_parts_for(const IcStepBatch& b, const IcAttention& a, int* part_len) const {
+        if (!meta.attention_counters) { if (part_len) *part_len = 0; return 1; }     // no counters: no cut
         int keys = b.max_position + 1;
         if (a.window > 0 && a.window + ic_attn_prefill_tile_rows() < keys) keys = a.window + ic_attn_prefill_tile_rows();
         return ic_attn_prefill_parts(b.n_prefill_tiles, a.n_heads, a.head_dim, keys, meta.compute_units, part_len);
@@ -92,7 +141,7 @@ struct IcDecoder {
         w.attn_out = take(T * (size_t)max_attn_width * ds);
         w.mixer_out = take(T * d * ds);
         w.ffn_out = take(T * d * ds);
-        const size_t few = std::min<size_t>(T, kFewRows);
+        const size_t few = std::min<size_t>(T, (size_t)ic_rule_few_rows());
         w.mixer_tail = take(few * d * 2);
         w.mixer_sumsq = take((size_t)parts * 16 * 4);
         w.ffn_tail = take(few * d * 2);
@@ -110,10 +159,10 @@ struct IcDecoder {
         w.part_ml = take(ml * 4);
         w.head_in = take((size_t)b.n_want * d * ds);
         size_t slices = 0;           // the O and down products as slices over K, where that pays
-        if (meta.dtype == IC_BF16 && T <= kMidRows)
-            for (const IcLayer& l : layers)
-                for (const int K : {l.attention.n_heads * l.attention.head_dim, l.ffn.intermediate})
-                    if (ic_gemm_splitk_pays(T, meta.hidden, K)) slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, K));
+        for (const IcLayer& l : layers)
+            for (const int K : {l.attention.n_heads * l.attention.head_dim, l.ffn.intermediate})
+                if (ic_rule_tail(meta.dtype, (int)T, meta.hidden, K, K, K) == IC_TAIL_SLICES)
+                    slices = std::max(slices, (size_t)ic_gemm_splitk_slices(meta.hidden, K));
         w.tail_parts = take(slices * T * d * 4);
         size_t cut = 0;              // the states of prompt tiles whose walk over the keys is cut into parts
         if (meta.dtype == IC_BF16 && b.n_prefill_tiles > 0)
@@ -129,7 +178,7 @@ struct IcDecoder {
     // out[M, N] = alpha * a w^T: the few-row product, or the library's.
     int linear(const void* a, int lda, const void* w, void* out, int out_dtype, int M, int N, int K, float alpha,
                const Deferred* rows, void* lib_ws, long long lib_ws_bytes, hipStream_t stream) const {
-        if (meta.dtype == IC_BF16 && M <= kFewRows) {
+        if (ic_rule_own_product(meta.dtype, meta.dtype, out_dtype, M)) {
             IcRowFactor rf{};
             if (rows) rf = IcRowFactor{rows->sumsq, rows->parts, rows->width, rows->eps};
             return ic_gemm_nt(a, IC_BF16, w, IC_BF16, out, out_dtype, M, N, K, lda, K, N, alpha, 0, rows ? &rf : nullptr,
@@ -140,19 +189,14 @@ struct IcDecoder {
     }
 
     // 17..64 rows (and 13..16 long ones) into the residual stream: x += alpha * (a w^T), out = rmsnorm(x) * weight, through the sliced
-    // product when it pays.  Returns 1 when done, 0 when the caller has to take the other way, < 0 on a fault.
+    // product and the kernel that sums the slices.
     int tail_in_slices(const void* a, int K, const void* w, float* parts, float* x, float alpha, const float* weight, float eps,
-                       void* out, int T, hipStream_t stream, int* status) const {
+                       void* out, int T, hipStream_t stream) const {
         const int d = meta.hidden;
-        *status = IC_OK;
-        if (meta.dtype != IC_BF16 || T > kMidRows || d % 4 || !ic_gemm_splitk_supported(T, d, K, K, K) ||
-            !ic_gemm_splitk_pays(T, d, K))
-            return 0;
         const int slices = ic_gemm_splitk_slices(d, K);
-        *status = ic_gemm_splitk(a, w, parts, T, d, K, K, K, slices, stream);
-        if (*status) return -1;
-        *status = ic_splitk_add_rmsnorm(parts, slices, T, x, alpha, weight, out, d, eps, stream);
-        return *status ? -1 : 1;
+        const int st = ic_gemm_splitk(a, w, parts, T, d, K, K, K, slices, stream);
+        if (st) return st;
+        return ic_splitk_add_rmsnorm(parts, slices, T, x, alpha, weight, out, d, eps, stream);
     }
 
     int forward(const IcStepBatch& b, void* workspace, long long workspace_bytes, void* lib_ws, long long lib_ws_bytes,
@@ -170,9 +214,7 @@ struct IcDecoder {
         void* normed = base + ws.normed;
         void* qkv = base + ws.qkv;
         void* attn_out = base + ws.attn_out;
-        const bool few = dt == IC_BF16 && T <= kFewRows;
         const int parts = ic_gemm_nt_residual_parts(d);
-        const bool can_split_norm = few && parts <= kMaxSumsqParts;
         int st;
 
         st = ic_embed(b.tokens, meta.embed_table, dt, x, T, d, meta.embed_scale, stream);
@@ -215,9 +257,7 @@ struct IcDecoder {
             const int* slots = b.group_slots[e.group];
             if (A.rot_dim > 0 && b.max_position >= A.max_positions) return fail(IC_ERR_ARG, "a position beyond the rotary tables", i);
             if (nkv > 0 && !slots) return fail(IC_ERR_ARG, "the cache slots of the entry's group", i);
-            // (up to 16 rows, or up to 32 where the weights can be read in whole cache lines and no row factors are owed)
-            const bool fused_qkv = dt == IC_BF16 && nkv > 0 && A.rot_dim == A.head_dim && ic_gemm_qkv_rope_supported(IC_BF16, A.head_dim) &&
-                                   (few || (!h_def && T <= ic_gemm_nt_epilogue_rows(2, d, d, d)));
+            const bool fused_qkv = ic_rule_qkv_fused(dt, T, d, d, d, A.head_dim, A.rot_dim, nkv, h_def != nullptr) != 0;
             IcRowFactor rf{};
             if (h_def) rf = IcRowFactor{h_def->sumsq, h_def->parts, h_def->width, h_def->eps};
             if (fused_qkv) {
@@ -239,12 +279,10 @@ struct IcDecoder {
             const int* tables = b.group_tables[e.group];
             const int bts = b.group_table_stride[e.group];
             const int ow = A.n_heads * A.head_dim;
-            const bool dec_ok = ic_attn_decode_supported(dt, A.head_dim) != 0;
-            const bool pre_ok = ic_attn_prefill_supported(dt, A.head_dim, ps) != 0;
             const int n_dec = b.n_decode_rows, n_tiles = b.n_prefill_tiles;
-            const bool use_dec = dec_ok && n_dec > 0 && (pre_ok || n_tiles == 0);
-            const bool use_pre = pre_ok && n_tiles > 0 && (dec_ok || n_dec == 0);
-            if (!((use_dec || n_dec == 0) && (use_pre || n_tiles == 0))) {
+            const int attn = ic_rule_attention(dt, A.head_dim, ps, n_dec, n_tiles);
+            const bool use_dec = (attn & IC_ATTN_SINGLE_TOKENS) != 0, use_pre = (attn & IC_ATTN_PORTIONS) != 0;
+            if (attn == IC_ATTN_GENERAL) {
                 st = ic_attn_generic(qkv, width, attn_out, ow, dt, e.k_cache, e.v_cache, tables, bts, b.token_req, b.positions, T,
                                      A.n_heads, A.n_kv_heads, A.head_dim, ps, A.softmax_scale, A.window, stream);
                 if (st) return fail(st, "attention (general kernel)", i);
@@ -263,7 +301,8 @@ struct IcDecoder {
                     st = ic_attn_prefill_split(qkv, width, attn_out, ow, dt, e.k_cache, e.v_cache, tables, bts, b.prefill_tiles,
                                                n_tiles, A.n_heads, A.n_kv_heads, A.head_dim, ps, A.softmax_scale, A.window, 0, parts,
                                                part_len, (float*)(base + ws.tile_parts),
-                                               ic_attn_prefill_scratch_floats(n_tiles, A.n_heads, A.head_dim, parts), stream);
+                                               ic_attn_prefill_scratch_floats(n_tiles, A.n_heads, A.head_dim, parts),
+                                               meta.attention_counters, stream);
                     if (st) return fail(st, "attention of prompt portions", i);
                 }
             }
@@ -271,11 +310,12 @@ struct IcDecoder {
             // ---- O projection, residual add, norm before the feed-forward --------------------------------
             Deferred mid;
             const Deferred* g_def = nullptr;
-            const int sliced = tail_in_slices(attn_out, ow, A.w_o, (float*)(base + ws.tail_parts), x, L.residual_scale, L.ffn_norm.weight,
-                                              L.ffn_norm.eps, normed, T, stream, &st);
-            if (sliced < 0) return fail(st, "the O product in slices with residual add and norm", i);
-            if (sliced) {
-            } else if (can_split_norm) {
+            const int o_tail = ic_rule_tail(dt, T, d, ow, ow, ow);
+            if (o_tail == IC_TAIL_SLICES) {
+                st = tail_in_slices(attn_out, ow, A.w_o, (float*)(base + ws.tail_parts), x, L.residual_scale, L.ffn_norm.weight,
+                                    L.ffn_norm.eps, normed, T, stream);
+                if (st) return fail(st, "the O product in slices with residual add and norm", i);
+            } else if (o_tail == IC_TAIL_SPLIT_NORM) {
                 IcResidualNorm tail{x, d, L.ffn_norm.weight, L.residual_scale, (float*)(base + ws.mixer_sumsq), parts};
                 st = ic_gemm_nt(attn_out, IC_BF16, A.w_o, IC_BF16, base + ws.mixer_tail, IC_BF16, T, d, ow, ow, ow, d, 1.0f, 2, nullptr,
                                 &tail, stream);
@@ -293,7 +333,7 @@ struct IcDecoder {
             // ---- feed-forward ----------------------------------------------------------------------------------
             const int di = L.ffn.intermediate;
             void* act = base + ws.act;
-            if (few || (dt == IC_BF16 && !g_def && T <= ic_gemm_nt_epilogue_rows(1, d, d, d))) {      // (up to 32 rows with whole-line loads)
+            if (ic_rule_gate_up_fused(dt, T, d, d, d, g_def != nullptr)) {
                 IcRowFactor gf{};
                 if (g_def) gf = IcRowFactor{g_def->sumsq, g_def->parts, g_def->width, g_def->eps};
                 st = ic_gemm_nt(g, IC_BF16, L.ffn.w_gate_up, IC_BF16, act, IC_BF16, T, 2 * di, d, d, d, di, 1.0f, 1, g_def ? &gf : nullptr,
@@ -305,12 +345,13 @@ struct IcDecoder {
                 st = ic_swiglu(base + ws.gate_up, act, dt, T, di, stream);
                 if (st) return fail(st, "SwiGLU", i);
             }
-            const int sliced_down = !succ ? 0 : tail_in_slices(act, di, L.ffn.w_down, (float*)(base + ws.tail_parts), x, L.residual_scale,
-                                                               succ_weight, succ->eps, normed, T, stream, &st);
-            if (sliced_down < 0) return fail(st, "the down product in slices with residual add and norm", i);
-            if (sliced_down) {
+            const int down_tail = succ ? ic_rule_tail(dt, T, d, di, di, di) : IC_TAIL_PLAIN;
+            if (down_tail == IC_TAIL_SLICES) {
+                st = tail_in_slices(act, di, L.ffn.w_down, (float*)(base + ws.tail_parts), x, L.residual_scale, succ_weight, succ->eps,
+                                    normed, T, stream);
+                if (st) return fail(st, "the down product in slices with residual add and norm", i);
                 owed = NORMED;
-            } else if (succ && can_split_norm) {
+            } else if (down_tail == IC_TAIL_SPLIT_NORM) {
                 IcResidualNorm tail{x, d, succ_weight, L.residual_scale, (float*)(base + ws.ffn_sumsq), parts};
                 st = ic_gemm_nt(act, IC_BF16, L.ffn.w_down, IC_BF16, base + ws.ffn_tail, IC_BF16, T, d, di, di, di, d, 1.0f, 2, nullptr,
                                 &tail, stream);
@@ -467,12 +508,6 @@ namespace {
 
 inline long long align4(long long n) { return (n + 3) & ~3LL; }
 
-int context_bucket(int n_keys) {      // key counts are rounded up to a power of two (at least 256) before the split is chosen
-    int b = 256;
-    while (b < n_keys) b *= 2;
-    return b;
-}
-
 struct HostLayout {
     long long tokens, positions, token_req, want_rows, decode_rows, tiles, slots[IC_MAX_CACHE_GROUPS], tables[IC_MAX_CACHE_GROUPS], total;
     int n_want, n_decode, n_tiles, stride[IC_MAX_CACHE_GROUPS];
@@ -577,7 +612,7 @@ IC_EXPORT int ic_decoder_pack(const IcDecoder* decoder, const IcHostBatch* batch
     s.want_rows_identity = identity ? 1 : 0;
     s.decode_rows_identity = (int)dec.size() == b.n_tokens ? 1 : 0;
     s.max_position = max_pos;
-    s.max_context = max_ctx ? context_bucket(max_ctx) : 0;
+    s.max_context = max_ctx ? ic_rule_context_bucket(max_ctx) : 0;
     s.fixed_decode_splits = b.fixed_decode_splits;
     s.tokens = device_ints + h.tokens; s.positions = device_ints + h.positions; s.token_req = device_ints + h.token_req;
     s.want_rows = device_ints + h.want_rows; s.decode_rows = device_ints + h.decode_rows; s.prefill_tiles = device_ints + h.tiles;

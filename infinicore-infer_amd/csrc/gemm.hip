@@ -20,6 +20,7 @@
 // 16x16x32 layout (lane l): A[i = l%16][k = 8(l/16)..+7], B[k = 8(l/16)..+7][j = l%16],
 // D[i = 4(l/16) + e][j = l%16], e = 0..3.
 #include "common.h"
+#include "infinicore_infer_variants.h"
 #include <utility>
 
 typedef short v4s __attribute__((ext_vector_type(4)));
@@ -445,10 +446,19 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         }
 }
 
-// Whole-line weight loads (LINES) where the sizes allow: 1 (the default) on, 0 off (for measurements and tests).
-static int g_lines_enabled = 1;
-IC_EXPORT int ic_gemm_nt_lines_enable(int on) { g_lines_enabled = on ? 1 : 0; return IC_OK; }
-static inline bool lines_apply(bool aligned, int K) { return aligned && g_lines_enabled && K % 64 == 0; }
+// What a caller of the *_variant entry points (tests and sweeps) asks for.  It holds for that one call on the calling
+// thread and changes nothing for any other call: no setting outlives the call that made it.
+struct Variant {
+    int lines = 1;             // whole-line weight loads (LINES) where the sizes allow; 0: loads in operand layout
+    int rope_tile_rows = 0;    // used weight rows per tile of ic_gemm_qkv_rope (16, 8, 4); 0: chosen from the number of heads
+};
+static thread_local Variant t_variant;
+struct VariantScope {
+    Variant saved;
+    explicit VariantScope(const Variant& v) : saved(t_variant) { t_variant = v; }
+    ~VariantScope() { t_variant = saved; }
+};
+static inline bool lines_apply(bool aligned, int K) { return aligned && t_variant.lines && K % 64 == 0; }
 
 template <typename TC, int NT, int MT, int WPB, int UNROLL, int EPI = 0, bool OWN_K = false, int AG = 1>
 static void launch_gemm(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw,
@@ -689,10 +699,6 @@ gemm_wide_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__ W,
     }
 }
 
-static bool g_wide_enabled = true;
-// For measurements: 0 sends wide products through the tiled kernel again.  Returns the previous setting.
-IC_EXPORT int ic_gemm_nt_wide_enable(int on) { const int was = g_wide_enabled; g_wide_enabled = on != 0; return was; }
-
 // false when the wide kernel does not take the shape.
 template <typename TC>
 static bool launch_gemm_wide(const void* A, const void* W, void* C, int M, int N, int K, int lda, int ldw, int ldc,
@@ -700,7 +706,7 @@ static bool launch_gemm_wide(const void* A, const void* W, void* C, int M, int N
     const int steps = (K + 31) / 32, groups = (steps + kWideDepth - 1) / kWideDepth;
     const int a_stride = groups * kWideDepth * 32 + 16;
     const size_t rows_bytes = (size_t)M * a_stride * 2;
-    const bool lines = g_lines_enabled && K >= 2048 && K % 64 == 0 && ldw % 64 == 0 && ((uintptr_t)W & 127) == 0;
+    const bool lines = t_variant.lines && K >= 2048 && K % 64 == 0 && ldw % 64 == 0 && ((uintptr_t)W & 127) == 0;
     auto lds_of = [&](int wv) { return rows_bytes + (4 * wv * 16 + 16) * sizeof(float) + (size_t)wv * (lines ? 16 * kLineRowBytes : 64 * 16); };
     // two blocks of 8 waves a compute unit; with many or long token rows one block of 16 waves, or of 8 when only that fits
     const bool two = 2 * lds_of(8) <= (size_t)kWideLdsLimit;
@@ -742,7 +748,7 @@ static void dispatch_gemm(const void* A, const void* W, void* C, int M, int N, i
     const int tiles = (N + 15) / 16;
 #define IC_GO(NT, MT, WPB, UN) launch_gemm<TC, NT, MT, WPB, UN>(A, W, C, M, N, K, lda, ldw, ldc, alpha, aligned, nf, stream)
     // tilings from a sweep over the projection shapes of 1B..8B models on MI355X
-    if (M <= 16 && tiles >= 2048 && aligned && g_wide_enabled &&
+    if (M <= 16 && tiles >= 2048 && aligned &&
         launch_gemm_wide<TC>(A, W, C, M, N, K, lda, ldw, ldc, alpha, nf, stream)) return;
     if (M <= 16) {
         if (tiles < 400) IC_GO(1, 1, 16, 4);
@@ -913,14 +919,6 @@ IC_EXPORT int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype,
 // dh a multiple of 32.  W: [(nh + 2 nkvh) * dh, K].
 IC_EXPORT int ic_gemm_qkv_rope_supported(int dtype, int dh) { return dtype == IC_BF16 && dh >= 32 && dh % 32 == 0; }
 
-// For tuning and tests: the used rows per tile of ic_gemm_qkv_rope (16, 8 or 4; 0: chosen from the number of heads).
-static int g_rope_tile_rows = 0;
-IC_EXPORT int ic_gemm_qkv_rope_tile_rows(int rows) {
-    if (rows != 0 && rows != 4 && rows != 8 && rows != 16) return IC_ERR_ARG;
-    g_rope_tile_rows = rows;
-    return IC_OK;
-}
-
 IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc,
                                const int* positions, const int* slots, const float* cos_t, const float* sin_t,
                                void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size,
@@ -937,7 +935,7 @@ IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int
     // (measured: 80 blocks on 256 units 7.6 -> 6.9 us with 8 rows; 144 blocks 16.1 -> 19.6, slower).
     const int pairs16 = (nh + 2 * nkvh) * (dh / 32), cus = compute_units();
     int rr = 16;
-    if (g_rope_tile_rows) rr = g_rope_tile_rows;
+    if (t_variant.rope_tile_rows) rr = t_variant.rope_tile_rows;
     else if (5 * pairs16 < 2 * cus) rr = (6 * pairs16 <= cus) ? 4 : 8;
     const RopeEpilogue rope{positions, slots, cos_t, sin_t, kcache, vcache, nh, nkvh, dh, page_size, rr};
     const int N = (nh + 2 * nkvh) * dh;
@@ -966,4 +964,26 @@ IC_EXPORT int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int
     else IC_ROPE(8, 4, false);
 #undef IC_ROPE
     return ic_launch_status();
+}
+
+// ---- the same entry points with a variant named by the caller (tests and sweeps; see infinicore_infer_variants.h) ----------
+IC_EXPORT int ic_gemm_nt_variant(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K,
+                                 int lda, int ldw, int ldc, float alpha, int c_mode, const IcRowFactor* row_factor,
+                                 const IcResidualNorm* tail, int whole_lines, hipStream_t stream) {
+    Variant v;
+    v.lines = whole_lines ? 1 : 0;
+    VariantScope scope(v);
+    return ic_gemm_nt(A, a_dtype, W, w_dtype, C, c_dtype, M, N, K, lda, ldw, ldc, alpha, c_mode, row_factor, tail, stream);
+}
+
+IC_EXPORT int ic_gemm_qkv_rope_variant(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc,
+                                       const int* positions, const int* slots, const float* cos_t, const float* sin_t,
+                                       void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size,
+                                       const IcRowFactor* row_factor, int tile_rows, hipStream_t stream) {
+    if (tile_rows != 0 && tile_rows != 4 && tile_rows != 8 && tile_rows != 16) return IC_ERR_ARG;
+    Variant v;
+    v.rope_tile_rows = tile_rows;
+    VariantScope scope(v);
+    return ic_gemm_qkv_rope(A, W, C, M, K, lda, ldw, ldc, positions, slots, cos_t, sin_t, kcache, vcache, nh, nkvh, dh, page_size,
+                            row_factor, stream);
 }

@@ -272,13 +272,11 @@ bool splits_ok(const float* P, int S, int M, int N) {
 
 }  // namespace
 
-// For measurements: 0 makes every block walk its slice from the start (1, the default: rotated starts).
-static int g_sk_rotate = 1;
-IC_EXPORT int ic_gemm_splitk_rotate(int on) { g_sk_rotate = on ? 1 : 0; return IC_OK; }
-
-// 1 when the sliced product takes these sizes: 1..64 rows of bfloat16, K a multiple of 8, aligned operands.
+// 1 when the sliced product takes these sizes: 1..64 rows of bfloat16, K a multiple of 8 and at least 64 (a lane's
+// clamped load of a weight row's last chunk starts up to 56 elements into the row: shorter rows would be read past
+// their end), aligned operands.
 IC_EXPORT int ic_gemm_splitk_supported(int M, int N, int K, int lda, int ldw) {
-    return M >= 1 && M <= 64 && N >= 1 && K >= 8 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K;
+    return M >= 1 && M <= 64 && N >= 1 && K >= 64 && K % 8 == 0 && lda % 8 == 0 && ldw % 8 == 0 && lda >= K && ldw >= K;
 }
 
 // Slices of K to use: blocks for about 7/8 of the compute units (beyond the units a second, part-filled round was
@@ -304,12 +302,9 @@ IC_EXPORT int ic_gemm_splitk_slices(int N, int K) {
 // 16 KB and more (from 9 rows on it loads its token operand once per k-step: the 8B shape's down projection takes 34 us
 // at 16 rows, the slices and the kernel that sums them 27.5; a decode step of that shape 4.06 -> 3.95 ms at batch 16,
 // 3.76 -> 3.76 at 12, 3.64 -> 3.69 at 9).
-static int g_sk_few_rows = 1;
-// For measurements: 0 leaves products of up to 16 rows to the few-row kernel throughout.
-IC_EXPORT int ic_gemm_splitk_few_rows(int on) { const int was = g_sk_few_rows; g_sk_few_rows = on != 0; return was; }
 IC_EXPORT int ic_gemm_splitk_pays(int M, int N, int K) {
     if (M <= 0 || M > 64 || N <= 0 || K <= 0 || N > 8192) return 0;
-    if (M <= 16 && (M <= 12 || K < 8192 || !g_sk_few_rows)) return 0;
+    if (M <= 16 && (M <= 12 || K < 8192)) return 0;
     const int col_blocks = (N + kSkCols - 1) / kSkCols;
     return 2 * col_blocks * ic_gemm_splitk_slices(N, K) >= compute_units_sk();
 }
@@ -325,10 +320,10 @@ IC_EXPORT int ic_gemm_splitk(const void* A, const void* W, float* P, int M, int 
     dim3 grid((N + kSkCols - 1) / kSkCols, n_slices), block(kSkThreads);
     const uint16_t* a = (const uint16_t*)A;
     const uint16_t* w = (const uint16_t*)W;
-    if (M <= 16) hipLaunchKernelGGL(gemm_splitk_kernel<1>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
-    else if (M <= 32) hipLaunchKernelGGL(gemm_splitk_kernel<2>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
-    else if (M <= 48) hipLaunchKernelGGL(gemm_splitk_kernel<3>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
-    else hipLaunchKernelGGL(gemm_splitk_kernel<4>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, g_sk_rotate);
+    if (M <= 16) hipLaunchKernelGGL(gemm_splitk_kernel<1>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, 1);
+    else if (M <= 32) hipLaunchKernelGGL(gemm_splitk_kernel<2>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, 1);
+    else if (M <= 48) hipLaunchKernelGGL(gemm_splitk_kernel<3>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, 1);
+    else hipLaunchKernelGGL(gemm_splitk_kernel<4>, grid, block, 0, stream, a, w, P, M, N, K, lda, ldw, per, 1);
     return ic_launch_status();
 }
 

@@ -86,6 +86,8 @@ typedef struct {
     const void* head_weight; // [vocab, hidden]
     IcNorm final_norm;
     const float* final_norm_scaled;   // final_norm.weight * logit_scale
+    int* attention_counters;          // ic_attn_prefill_counter_ints() ints of the caller's, zero when the decoder is made; every step
+                                      // leaves them zero.  Steps that overlap in time (two streams) need decoders with counters of their own
 } IcDecoderMeta;
 
 // A step's batch where it lies on the device.  Tokens of all requests are concatenated in request order.
@@ -149,6 +151,34 @@ int ic_decoder_step(IcDecoder* decoder, const IcHostBatch* batch, int* staging, 
 // ic_decoder_pack only lays the batch out (no GPU call); the caller copies staging[0 .. n_ints) to device_ints.
 int ic_decoder_pack(const IcDecoder* decoder, const IcHostBatch* batch, int* staging, const int* device_ints,
                     long long n_ints, IcStepBatch* laid_out);
+
+// ---- which kernel takes what ------------------------------------------------------------------------------------------
+// The rules by which a step's products and attention choose their kernels.  ic_decoder_forward asks them, and so
+// does whoever issues the same kernels one by one (the parts' Python forward), so that both launch the same kernels
+// for the same step and a rule is written once.  `dtype`: the compute dtype; lda, ldw: row strides in elements.
+#define IC_TAIL_PLAIN 0       // the product, then the add+norm kernel
+#define IC_TAIL_SPLIT_NORM 1  // the few-row product adds to the residual stream and hands on x * weight and sums of squares
+#define IC_TAIL_SLICES 2      // slices over K, then the kernel that sums them, adds and applies the whole norm
+#define IC_ATTN_GENERAL 0     // the general kernel for every row
+#define IC_ATTN_SINGLE_TOKENS 1   // (bit) the split-key kernel for rows that are a request's single new token
+#define IC_ATTN_PORTIONS 2        // (bit) the tiled matrix-core kernel for prompt portions
+int ic_rule_few_rows();           // rows up to which the package's own product runs instead of the library's
+int ic_rule_sumsq_parts_max();    // column blocks of sums of squares a product takes as row factors
+// 1: a plain product of `rows` rows runs in the package's own kernel (ic_gemm_nt), 0: in the library (ic_matmul).
+int ic_rule_own_product(int a_dtype, int w_dtype, int c_dtype, int rows);
+// 1: the QKV projection runs with rotary and cache write in its epilogue (ic_gemm_qkv_rope); 0: product, then ic_rope_kv_write.
+// kv_heads_written: 0 when the entry writes no cache; row_factors_owed: the rows' norm is half done (IcRowFactor).
+int ic_rule_qkv_fused(int dtype, int rows, int K, int lda, int ldw, int head_dim, int rot_dim, int kv_heads_written, int row_factors_owed);
+// 1: the gate/up projection runs with SwiGLU in its epilogue (ic_gemm_nt, c_mode 1); 0: product, then ic_swiglu.
+int ic_rule_gate_up_fused(int dtype, int rows, int K, int lda, int ldw, int row_factors_owed);
+// How a projection into the residual stream (O, down: N = hidden) that a norm follows runs: IC_TAIL_*.
+int ic_rule_tail(int dtype, int rows, int N, int K, int lda, int ldw);
+// Which attention kernels a step with n_decode_rows single-token rows and n_tiles prompt tiles takes: IC_ATTN_GENERAL, or bits.
+int ic_rule_attention(int dtype, int head_dim, int page_size, int n_decode_rows, int n_tiles);
+// Key counts are rounded up before the key split of single-token rows is chosen, so that a recorded step serves a range
+// of lengths and splits as an eager one does: to a power of two up to 1,024 (at least 256), above that to a multiple of
+// a quarter of the power of two below (2,560, 3,072, 3,584, 4,096, 5,120 ...).
+int ic_rule_context_bucket(int n_keys);
 
 // How many ways to split the keys of single-token rows (from sweeps on MI355X with caches that do not fit the
 // last-level cache); see the decode attention kernel.  elem_bytes: of a cache element.  matrix_cores: 1 when the

@@ -52,10 +52,13 @@ int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int out_strid
 // The same with a query tile's walk over the keys cut into parts that run as blocks of their own (one wave group): the grid holds
 // `parts` blocks per (tile, head), a part walks at least part_len key tiles of 64, the block that arrives last merges the parts
 // through `scratch` (ic_attn_prefill_scratch_floats floats).  ic_attn_prefill_parts proposes parts and part_len for a step whose
-// longest tile sees max_keys keys (1: no cut).  Launches that cut and overlap in time on one device share the arrival counters: use one stream.
+// longest tile sees max_keys keys (1: no cut).  The parts count themselves in at `counters`: ic_attn_prefill_counter_ints() ints of
+// the caller's that are zero before the first launch; every launch leaves them zero, so one buffer serves all launches that follow
+// each other on a stream.  Launches that overlap in time (two streams) need counters of their own.
 long long ic_attn_prefill_scratch_floats(int n_tiles, int nh, int dh, int parts);
+int ic_attn_prefill_counter_ints();
 int ic_attn_prefill_parts(int n_tiles, int nh, int dh, int max_keys, int compute_units, int* part_len);
-int ic_attn_prefill_split(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, int parts, int part_len, float* scratch, long long scratch_floats, hipStream_t stream);
+int ic_attn_prefill_split(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, int parts, int part_len, float* scratch, long long scratch_floats, int* counters, hipStream_t stream);
 
 // ---- gemm.hip ---------------------------------------------------------------------------------------
 // A norm y = x * rsqrt(mean(x^2) + eps) * w between two products of M <= 16 rows can be split over them: the
@@ -82,22 +85,12 @@ typedef struct {
 int ic_gemm_nt_supported(int a_dtype, int w_dtype, int c_dtype);
 int ic_gemm_nt_residual_parts(int N);
 int ic_gemm_nt(const void* A, int a_dtype, const void* W, int w_dtype, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int c_mode, const IcRowFactor* row_factor, const IcResidualNorm* tail, hipStream_t stream);
-// Products of up to 16 rows with 32,768 weight rows or more (the output head) run in a kernel whose waves own whole
-// weight tiles; 0 sends them through the tiled kernel instead (for measurements).  Returns the previous setting.
-int ic_gemm_nt_wide_enable(int on);
-// 1 (the default): with K a multiple of 64 and aligned operands the few-row products read their weights in whole cache lines
-// (8 rows x 128 bytes a wave load, not kept in the caches) and pass them through LDS into operand layout; 0: loads in operand layout.
-int ic_gemm_nt_lines_enable(int on);
 // Rows that the products with an epilogue take: kind 1 (c_mode 1, SwiGLU) and kind 2 (ic_gemm_qkv_rope) 32 where the weights can be
 // read in whole cache lines (K a multiple of 64, row strides multiples of 8), 16 otherwise; without row factors above 16 rows.
 int ic_gemm_nt_epilogue_rows(int kind, int K, int lda, int ldw);
-// The same with the tiling chosen by the caller (tuning and tests); nt == 0 selects the SwiGLU variant.
-int ic_gemm_nt_cfg(const void* A, const void* W, void* C, int c_dtype, int M, int N, int K, int lda, int ldw, int ldc, float alpha, int nt, int wpb, int unroll, hipStream_t stream);
 // QKV projection of M <= 16 rows with rotary and cache write in the epilogue; row_factor nullable.
 int ic_gemm_qkv_rope_supported(int dtype, int dh);
 int ic_gemm_qkv_rope(const void* A, const void* W, void* C, int M, int K, int lda, int ldw, int ldc, const int* positions, const int* slots, const float* cos_t, const float* sin_t, void* kcache, void* vcache, int nh, int nkvh, int dh, int page_size, const IcRowFactor* row_factor, hipStream_t stream);
-// For tuning and tests: used weight rows per tile of ic_gemm_qkv_rope (16, 8 or 4; 0: chosen from the number of heads).
-int ic_gemm_qkv_rope_tile_rows(int rows);
 
 // ---- gemm_splitk.hip ----------------------------------------------------------------------------------
 // Products of 1..64 rows (bfloat16) as float32 slices over K, P[s, m, n] = A[m, K_s] . W[n, K_s], and the kernel
@@ -106,8 +99,6 @@ int ic_gemm_qkv_rope_tile_rows(int rows);
 int ic_gemm_splitk_supported(int M, int N, int K, int lda, int ldw);
 int ic_gemm_splitk_slices(int N, int K);      // how many slices to use (never an empty one)
 int ic_gemm_splitk_pays(int M, int N, int K);
-int ic_gemm_splitk_rotate(int on);            // for measurements: 0 = every block walks its slice of K from the start (default 1: rotated starts)
-int ic_gemm_splitk_few_rows(int on);          // for measurements: 0 = products of up to 16 rows never run in slices (default 1: 13..16 rows of 16 KB and more do)
 int ic_gemm_splitk(const void* A, const void* W, float* P, int M, int N, int K, int lda, int ldw, int n_slices, hipStream_t stream);
 // P [S, M, d]: x += alpha * (the product, rounded to bfloat16); out = rmsnorm(x) * w.
 int ic_splitk_add_rmsnorm(const float* P, int n_slices, int M, float* x, float alpha, const float* w, void* out, int d, float eps, hipStream_t stream);

@@ -42,6 +42,21 @@ class Workspace:
         self._views[key] = (shape, view)
         return view
 
+    def zeroed(self, name: str, shape, dtype) -> torch.Tensor:
+        """A buffer of a fixed shape that is zero when it is first handed out and is the caller's to keep so (arrival
+        counters that every launch leaves at zero).  It is never regrown, so what it holds is never lost."""
+        key = (name, dtype)
+        shape = tuple(shape)
+        buf = self._bufs.get(key)
+        if buf is None:
+            if self.frozen:
+                raise RuntimeError("workspace buffer %r would have to be made, but recorded steps hold the workspace" % name)
+            buf = torch.zeros(shape, dtype=dtype, device=self.device)
+            self._bufs[key] = buf
+        elif tuple(buf.shape) != shape:
+            raise RuntimeError("workspace buffer %r has a fixed shape %s, asked for %s" % (name, tuple(buf.shape), shape))
+        return buf
+
     def bytes(self) -> int:
         return sum(b.numel() * b.element_size() for b in self._bufs.values())
 

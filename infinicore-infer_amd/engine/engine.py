@@ -35,17 +35,9 @@ def _align4(n: int) -> int:
 
 
 def _context_bucket(n_keys: int) -> int:
-    """Key counts are rounded up before the key split of single-token rows is chosen, so eager and
-    recorded steps split alike and a recorded graph serves a whole range of lengths: to a power of
-    two up to 1,024 (at least 256), above that to a quarter of the power of two below (2,560, 3,072,
-    3,584, 4,096, 5,120 ...), so that the count the split is chosen for is at most a quarter off."""
-    b = 256
-    while b < n_keys:
-        b *= 2
-    if b <= 1024:
-        return b
-    q = b // 8
-    return (n_keys + q - 1) // q * q
+    """The key count a step's key split is chosen for: the kernel library's rounding (one rule for steps issued from
+    here, for recorded ones and for the native step function, so that they split alike)."""
+    return ops.rule_context_bucket(n_keys)
 
 
 class _PinnedRing:
@@ -141,6 +133,8 @@ class Engine:
         self.graph_steps = 0         # steps that took the recorded path (the recording one included)
         self.graph_replays = 0       # of these, replays of an existing recording
         self.steps_ahead = 0         # recorded steps that took their tokens from the device (step_ahead)
+        self._sample_host = None     # pinned staging of the sampler's per-row parameters, and of its tokens
+        self._sampled_host = None
         self._ahead_out = None       # two sets of buffers for tokens sampled without waiting, used in turn
         self._ahead_turn = 0
         self.graphs_evicted = 0
@@ -218,6 +212,7 @@ class Engine:
                 try:
                     logits = self._graph_step(entries, starts)
                 except BaseException:
+                    self._forget_recorded_rows()
                     for e, p0 in zip(entries, starts):
                         self.cache.truncate(e.req_id, p0)
                     raise
@@ -277,6 +272,7 @@ class Engine:
                 with ops.stream_scope():
                     logits = self._eager_step(entries, starts)
         except BaseException:
+            self._forget_recorded_rows()
             for e in entries:
                 if e.req_id in new_ids:
                     if self.cache.has_request(e.req_id):
@@ -316,12 +312,29 @@ class Engine:
         try:
             logits = self._graph_step(entries, starts, device_tokens)
         except BaseException:
+            self._forget_recorded_rows()
             for e, p0 in zip(entries, starts):
                 self.cache.truncate(e.req_id, p0)
             raise
         self.steps_run += 1
         self.steps_ahead += 1
         return logits
+
+    def _forget_recorded_rows(self):
+        """After a step that failed: the pinned images of the recorded steps may hold block-table rows with pages that
+        the failed step took and that are given back now.  Such a row is rewritten only when its key (request, page
+        count, first live page) changes, and the same key can come back with another page; so every row is
+        written anew at its next use."""
+        for g in self._graphs.values():
+            g.forget_rows()
+
+    def _drop_native(self):
+        """The native step function cannot run this model's products (the library has no algorithm for one): from
+        now on the parts' forward steps it.  Recordings made around the native call, and the frozen workspace they
+        share, go with it."""
+        self.native = None
+        self._graphs.clear()
+        self._graph_ws = None
 
     def _append_single_tokens(self, entries):
         """The checks and the cache growth of a step in which every entry is an admitted request's single
@@ -370,7 +383,7 @@ class Engine:
                 self.native_steps += 1
                 return out
             except ops.NoLibraryAlgorithm:
-                self.native = None        # see _forward; nothing of the half-issued step is kept
+                self._drop_native()       # see _forward; nothing of the half-issued step is kept
         return self.model.forward(self._build_context(entries, starts))
 
     def _forward(self, ctx):
@@ -385,7 +398,7 @@ class Engine:
             except ops.NoLibraryAlgorithm:
                 # the library has no algorithm for a product of this step: the Python path knows a detour.
                 # Nothing of the half-issued step is kept (the residual stream is rebuilt, cache writes repeat).
-                self.native = None
+                self._drop_native()
         return self.model.forward(ctx)
 
     # ---- packing the batch ------------------------------------------------------------------------
@@ -604,10 +617,30 @@ class Engine:
             ops.argmax(logits, out, self.ws.buffer("argmax_val", (64 * R,), torch.float32),
                        self.ws.buffer("argmax_idx", (64 * R,), torch.int32))
         else:
-            f = torch.tensor([list(temperature), list(top_p), list(uniform)], dtype=torch.float32).to(self.device)
-            k = torch.tensor(list(top_k), dtype=torch.int32).to(self.device)
-            ops.sample(logits, out, f[0].contiguous(), k, f[1].contiguous(), f[2].contiguous())
-        return out.cpu().tolist()
+            # the rows' parameters go through pinned memory into workspace buffers: nothing is allocated per step
+            n = max(R, self.graph_max_batch, 1)
+            if self._sample_host is None or self._sample_host[0].shape[1] < R:
+                self._sample_host = (torch.empty(3, n, dtype=torch.float32, pin_memory=True),
+                                     torch.empty(n, dtype=torch.int32, pin_memory=True), torch.cuda.Event())
+                self._sample_host[2].record()
+            f_host, k_host, copied = self._sample_host
+            width = f_host.shape[1]
+            copied.synchronize()                        # the copies of the call before have read the pinned buffers
+            fa, ka = f_host.numpy(), k_host.numpy()
+            fa[0, :R], fa[1, :R], fa[2, :R] = temperature, top_p, uniform
+            ka[:R] = top_k
+            f = self.ws.buffer("sample_f", (3, width), torch.float32)
+            k = self.ws.buffer("sample_k", (width,), torch.int32)
+            f.copy_(f_host, non_blocking=True)
+            k.copy_(k_host, non_blocking=True)
+            copied.record()
+            ops.sample(logits, out, f[0, :R], k[:R], f[1, :R], f[2, :R])
+        host = self._sampled_host
+        if host is None or host.numel() < R:
+            host = self._sampled_host = torch.empty(max(R, self.graph_max_batch, 1), dtype=torch.int32, pin_memory=True)
+        host[:R].copy_(out, non_blocking=True)
+        torch.cuda.current_stream().synchronize()
+        return host[:R].tolist()
 
     def sample_ahead(self, logits, temperature=None, top_k=None, top_p=None, uniform=None):
         """As ``sample``, without waiting for the device: returns (the tokens on the device, int32 [rows], and a
@@ -634,8 +667,9 @@ class Engine:
             ops.argmax(logits, out, self.ws.buffer("argmax_val", (64 * R,), torch.float32),
                        self.ws.buffer("argmax_idx", (64 * R,), torch.int32))
         else:
-            b["f_host"][:, :R] = torch.tensor([list(temperature), list(top_p), list(uniform)], dtype=torch.float32)
-            b["k_host"][:R] = torch.tensor(list(top_k), dtype=torch.int32)
+            fa, ka = b["f_host"].numpy(), b["k_host"].numpy()
+            fa[0, :R], fa[1, :R], fa[2, :R] = temperature, top_p, uniform
+            ka[:R] = top_k
             b["f"].copy_(b["f_host"], non_blocking=True)        # (pinned: the host does not wait for the device)
             b["k"].copy_(b["k_host"], non_blocking=True)
             ops.sample(logits, out, b["f"][0, :R], b["k"][:R], b["f"][1, :R], b["f"][2, :R])
@@ -731,6 +765,12 @@ class _DecodeGraph:
                     a[base + len(table):base + self.maxb] = 0
                     self._row_keys[g][r] = key
         self.ctx.host_state_slots = slots
+
+    def forget_rows(self):
+        """Every block-table row of the pinned image is written anew at its next use."""
+        for keys in self._row_keys:
+            for r in range(len(keys)):
+                keys[r] = None
 
     def capture(self, engine):
         """Run the step once eagerly: that is the step's result, and every buffer then exists.  Then

@@ -57,6 +57,8 @@ class NativeDecoder:
             return None
         scaled_w = scaled.deferred()[0]
         lib = get_lib()
+        # arrival counters of the prompt attention's cut walks: this engine's own, zero now and after every step
+        counters = torch.zeros(ops.attention_prefill_counter_ints(), dtype=torch.int32, device=engine.device)
         layer_arr = (IcLayer * len(layers))(*layers)
         entries = []
         for e in model.schedule:
@@ -65,12 +67,12 @@ class NativeDecoder:
         entry_arr = (IcRunEntry * len(entries))(*entries)
         meta = IcDecoderMeta(ops.dtype_code(rt.dtype), model.spec.hidden_size, model.spec.vocab_size, engine.page_size,
                              len(layers), len(entries), len(engine.groups), engine.cu_count, emb[1], head[1], emb[0],
-                             head[0], fin, scaled_w.data_ptr())
+                             head[0], fin, scaled_w.data_ptr(), counters.data_ptr())
         handle = lib.ic_decoder_create(ctypes.byref(meta), layer_arr, entry_arr)
         if not handle:
             raise KernelError("the native step function refused the model: %s"
                               % lib.ic_decoder_create_error().decode())
-        return cls(handle, lib, model.spec.vocab_size, (layer_arr, entry_arr, meta, scaled_w))
+        return cls(handle, lib, model.spec.vocab_size, (layer_arr, entry_arr, meta, scaled_w, counters))
 
     def workspace_bytes_for_decode(self, n_requests: int) -> int:
         """Workspace bytes that any step of up to ``n_requests`` single tokens needs (with the most key

@@ -92,6 +92,10 @@ class Scheduler:
         # decoding one step ahead of the host: not together with kept caches (a cache would be kept with a token more)
         self.overlap = (bool(overlap) and not self.prefix_cache and hasattr(engine, "step_ahead")
                         and hasattr(engine, "sample_ahead") and getattr(engine, "use_graphs", True))
+        # rows a step may have to run ahead: what the engine records (a larger batch has no recording, so
+        # ``step_ahead`` would refuse it and ``sample_ahead`` has no buffers for it)
+        cap = getattr(engine, "graph_max_batch", None)
+        self._ahead_rows = (1 << 30) if cap is None else int(cap)
         self._ahead: Optional[_Ahead] = None
         self.n_ahead = 0                 # steps issued before the tokens of the step before were read
         self.idle: "OrderedDict[object, List[int]]" = OrderedDict()    # kept cache id -> the tokens it holds, oldest first
@@ -382,7 +386,7 @@ class Scheduler:
             return []
         positions = [self.cache.length(r.task.id) for r in samplers]
         if (self.overlap and not self.waiting and len(samplers) == len(self.running)
-                and all(r.decoding for r in self.running)):
+                and len(samplers) <= self._ahead_rows and all(r.decoding for r in self.running)):
             # every running request decodes from here on: do not wait for this step's tokens, the next call
             # issues the step after it first
             dev, wait = self.engine.sample_ahead(logits, *self._sampling_arguments(samplers, 0))

@@ -67,7 +67,8 @@ class IcRunEntry(_c.Structure):
 class IcDecoderMeta(_c.Structure):
     _fields_ = [("dtype", _I), ("hidden", _I), ("vocab", _I), ("page_size", _I), ("n_layers", _I), ("n_entries", _I),
                 ("n_groups", _I), ("compute_units", _I), ("embed_scale", _F), ("logit_scale", _F),
-                ("embed_table", _P), ("head_weight", _P), ("final_norm", IcNorm), ("final_norm_scaled", _P)]
+                ("embed_table", _P), ("head_weight", _P), ("final_norm", IcNorm), ("final_norm_scaled", _P),
+                ("attention_counters", _P)]
 
 
 class IcStepBatch(_c.Structure):
@@ -104,15 +105,15 @@ _SIGNATURES = {
     "ic_attn_prefill_groups": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ic_attn_prefill_scratch_floats": [_I, _I, _I, _I],
     "ic_attn_prefill_parts": [_I, _I, _I, _I, _I, _c.POINTER(_I)],
-    "ic_attn_prefill_split": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _LL, _P],
+    "ic_attn_prefill_split": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _LL, _P, _P],
+    "ic_attn_prefill_counter_ints": [],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
     "ic_argmax": [_P, _LL, _I, _I, _P, _P, _P, _P],
     "ic_argmax_static_max_rows": [],
     "ic_argmax_static": [_P, _LL, _I, _I, _P, _P],
     "ic_gemm_nt": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _P],
     "ic_gemm_nt_residual_parts": [_I],
-    "ic_gemm_nt_wide_enable": [_I],
-    "ic_gemm_nt_lines_enable": [_I],
+    "ic_gemm_nt_variant": [_P, _I, _P, _I, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _RF, _RN, _I, _P],
     "ic_gemm_nt_epilogue_rows": [_I, _I, _I, _I],
     "ic_peak_mfma_bf16": [_P, _I, _I, _P],
     "ic_peak_read": [_P, _LL, _I, _P, _P],
@@ -122,16 +123,22 @@ _SIGNATURES = {
     "ic_matmul_supported": [_I, _I],
     "ic_matmul": [_P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _P, _LL, _P],
     "ic_matmul_tune": [_P, _I, _P, _P, _I, _I, _I, _I, _I, _I, _I, _P, _LL, _P, _LL, _I, _P],
-    "ic_gemm_qkv_rope_tile_rows": [_I],
+    "ic_gemm_qkv_rope_variant": [_P, _P, _P, _I, _I, _I, _I, _I, _P, _P, _P, _P, _P, _P, _I, _I, _I, _I, _RF, _I, _P],
     "ic_gemm_nt_cfg": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _I, _F, _I, _I, _I, _P],
     "ic_attn_decode_splits": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
     "ic_gemm_splitk_supported": [_I, _I, _I, _I, _I],
     "ic_gemm_splitk_slices": [_I, _I],
     "ic_gemm_splitk": [_P, _P, _P, _I, _I, _I, _I, _I, _I, _P],
     "ic_gemm_splitk_pays": [_I, _I, _I],
-    "ic_gemm_splitk_rotate": [_I],
-    "ic_gemm_splitk_few_rows": [_I],
     "ic_splitk_add_rmsnorm": [_P, _I, _I, _P, _F, _P, _P, _I, _F, _P],
+    "ic_rule_few_rows": [],
+    "ic_rule_sumsq_parts_max": [],
+    "ic_rule_own_product": [_I, _I, _I, _I],
+    "ic_rule_qkv_fused": [_I, _I, _I, _I, _I, _I, _I, _I, _I],
+    "ic_rule_gate_up_fused": [_I, _I, _I, _I, _I, _I],
+    "ic_rule_tail": [_I, _I, _I, _I, _I, _I],
+    "ic_rule_attention": [_I, _I, _I, _I, _I],
+    "ic_rule_context_bucket": [_I],
     "ic_decoder_create": [_c.POINTER(IcDecoderMeta), _c.POINTER(IcLayer), _c.POINTER(IcRunEntry)],
     "ic_decoder_create_error": [],
     "ic_decoder_destroy": [_P],

@@ -257,31 +257,41 @@ def attention_prefill_parts(n_tiles: int, n_heads: int, head_dim: int, max_keys:
     return int(parts), int(part_len.value)
 
 
+def attention_prefill_counter_ints() -> int:
+    return int(get_lib().ic_attn_prefill_counter_ints())
+
+
 def attention_prefill_scratch_floats(n_tiles: int, n_heads: int, head_dim: int, parts: int) -> int:
     return int(get_lib().ic_attn_prefill_scratch_floats(int(n_tiles), int(n_heads), int(head_dim), int(parts)))
 
 
 def attention_prefill(q, out, kcache, vcache, block_tables, tiles, n_tiles, n_heads, n_kv_heads, head_dim,
                       page_size, scale: float, window: int = 0, groups: int = 0, parts: int = 1, part_len: int = 0,
-                      scratch=None):
+                      scratch=None, counters=None):
     """Matrix-core attention of prompt portions.  tiles: int32 [n, 4] rows of
     (request row in block_tables, first token row, rows <= tile_rows, first position).
     groups: wave groups per query tile (1 or 2); 0 lets the kernel choose from the number of blocks.
     parts > 1: every tile's walk over the keys is cut into up to ``parts`` blocks of at least ``part_len`` key tiles
-    that meet through ``scratch`` (float32, attention_prefill_scratch_floats(...) elements)."""
+    that meet through ``scratch`` (float32, attention_prefill_scratch_floats(...) elements) and count themselves in at
+    ``counters`` (int32, attention_prefill_counter_ints() elements, zero before the first launch; every launch leaves them
+    zero; launches that overlap in time need counters of their own)."""
     _need(groups in (0, 1, 2), "attention_prefill: groups must be 0, 1 or 2")
     _attn_common(q, out, kcache, vcache, block_tables, n_heads, n_kv_heads, head_dim, page_size)
     _need(tiles.dtype == torch.int32 and tiles.is_contiguous() and tiles.dim() == 2 and tiles.shape[1] == 4
           and tiles.shape[0] >= n_tiles, "attention_prefill: tiles must be int32 [n, 4]")
     if parts > 1:
         _dev(scratch)
+        _dev(counters)
         _need(scratch is not None and scratch.dtype == torch.float32 and scratch.is_contiguous(),
               "attention_prefill: a cut walk needs float32 scratch memory")
+        _need(counters is not None and counters.dtype == torch.int32 and counters.is_contiguous()
+              and counters.numel() >= attention_prefill_counter_ints(), "attention_prefill: a cut walk needs its int32 arrival counters")
     check(get_lib().ic_attn_prefill_split(
         q.data_ptr(), q.stride(0), out.data_ptr(), out.stride(0), dtype_code(q.dtype), kcache.data_ptr(),
         vcache.data_ptr(), block_tables.data_ptr(), block_tables.stride(0), tiles.data_ptr(), n_tiles,
         n_heads, n_kv_heads, head_dim, page_size, float(scale), int(window or 0), int(groups), int(parts), int(part_len),
-        scratch.data_ptr() if parts > 1 else None, scratch.numel() if parts > 1 else 0, _stream()),
+        scratch.data_ptr() if parts > 1 else None, scratch.numel() if parts > 1 else 0,
+        counters.data_ptr() if parts > 1 else None, _stream()),
         "attention_prefill")
 
 
@@ -338,7 +348,58 @@ def gemm_nt_supported(a_dtype, w_dtype, c_dtype) -> bool:
         return False
 
 
-MAX_SUMSQ_PARTS = 256      # column blocks of sums of squares a product can take as row factors
+# ---- which kernel takes what: the library's rules, shared with its native step function ----------------------------
+TAIL_PLAIN, TAIL_SPLIT_NORM, TAIL_SLICES = 0, 1, 2
+ATTN_GENERAL, ATTN_SINGLE_TOKENS, ATTN_PORTIONS = 0, 1, 2
+
+
+def _code_or_none(dt):
+    return _DT.get(dt)
+
+
+def rule_own_product(a_dtype, w_dtype, c_dtype, rows: int) -> bool:
+    """True when a plain product of ``rows`` rows runs in the package's own kernel (gemm_nt), not in the library."""
+    codes = (_code_or_none(a_dtype), _code_or_none(w_dtype), _code_or_none(c_dtype))
+    return None not in codes and bool(get_lib().ic_rule_own_product(codes[0], codes[1], codes[2], int(rows)))
+
+
+def rule_qkv_fused(dtype, rows: int, a, w, head_dim: int, rot_dim: int, kv_heads_written: int, row_factors_owed: bool) -> bool:
+    """True when the QKV projection of a[rows, K] with w runs with rotary and cache write in its epilogue."""
+    code = _code_or_none(dtype)
+    return code is not None and bool(get_lib().ic_rule_qkv_fused(code, int(rows), int(a.shape[1]), int(a.stride(0)), int(w.stride(0)),
+                                                                 int(head_dim), int(rot_dim), int(kv_heads_written),
+                                                                 int(bool(row_factors_owed))))
+
+
+def rule_gate_up_fused(dtype, rows: int, a, w, row_factors_owed: bool) -> bool:
+    """True when the gate/up projection of a[rows, K] with w runs with SwiGLU in its epilogue."""
+    code = _code_or_none(dtype)
+    return code is not None and bool(get_lib().ic_rule_gate_up_fused(code, int(rows), int(a.shape[1]), int(a.stride(0)),
+                                                                     int(w.stride(0)), int(bool(row_factors_owed))))
+
+
+def rule_tail(dtype, a, w) -> int:
+    """How the projection a w^T into the residual stream, followed by a norm, runs: TAIL_PLAIN, TAIL_SPLIT_NORM or TAIL_SLICES."""
+    code = _code_or_none(dtype)
+    if code is None or a.dtype != dtype or w.dtype != dtype:
+        return TAIL_PLAIN
+    return int(get_lib().ic_rule_tail(code, int(a.shape[0]), int(w.shape[0]), int(a.shape[1]), int(a.stride(0)), int(w.stride(0))))
+
+
+def rule_attention(dtype, head_dim: int, page_size: int, n_decode_rows: int, n_tiles: int) -> int:
+    """ATTN_GENERAL, or the bits ATTN_SINGLE_TOKENS and ATTN_PORTIONS: which attention kernels a step takes."""
+    return int(get_lib().ic_rule_attention(dtype_code(dtype), int(head_dim), int(page_size), int(n_decode_rows), int(n_tiles)))
+
+
+def rule_context_bucket(n_keys: int) -> int:
+    """The key count that the key split of single-token rows is chosen for (rounded up, so that a recorded step
+    serves a range of lengths and splits as an eager one does)."""
+    return int(get_lib().ic_rule_context_bucket(int(n_keys)))
+
+
+def max_sumsq_parts() -> int:
+    """Column blocks of sums of squares a product can take as row factors."""
+    return int(get_lib().ic_rule_sumsq_parts_max())
 
 
 def residual_parts(n: int) -> int:
@@ -354,7 +415,7 @@ def _row_factor(row_factor, M, what):
     _dev(sumsq)
     _need(M <= 16, what + ": row factors need at most 16 rows")
     _need(sumsq.dtype == torch.float32 and sumsq.is_contiguous() and sumsq.dim() == 2 and sumsq.shape[1] == 16
-          and 0 < sumsq.shape[0] <= MAX_SUMSQ_PARTS, what + ": sums of squares must be float32 [<= 256, 16]")
+          and 0 < sumsq.shape[0] <= max_sumsq_parts(), what + ": sums of squares must be float32 [<= 256, 16]")
     _need(width > 0, what + ": width")
     return IcRowFactor(sumsq.data_ptr(), sumsq.shape[0], int(width), float(eps))
 
@@ -365,14 +426,15 @@ def gemm_epilogue_rows(kind: str, a, w) -> int:
     return int(get_lib().ic_gemm_nt_epilogue_rows({"swiglu": 1, "rope": 2}[kind], int(a.shape[1]), int(a.stride(0)), int(w.stride(0))))
 
 
-def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_factor=None, residual=None):
+def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_factor=None, residual=None, whole_lines: bool = True):
     """out[M, N] = alpha * a[M, K] @ w[N, K]^T (bfloat16 operands, float32 accumulation).
     swiglu_output (M <= gemm_epilogue_rows("swiglu", a, w)): w = [gate rows; up rows] and out[M, N/2] = up * silu(gate).
     row_factor = (sumsq [n_parts, 16], width, eps), M <= 16: row m of the product is first multiplied by
     rsqrt(sumsq[:, m].sum() / width + eps), the factor an RMS norm of a's rows still owes.
     residual = (x float32 [M, N], weight float32 [N], beta, sumsq_out float32 [residual_parts(N), 16]),
     M <= 16, bfloat16 out: x += beta * (the product rounded to bfloat16); out = x * weight;
-    sumsq_out[b, m] = sum of x[m]^2 over columns 16 b .. 16 b + 15."""
+    sumsq_out[b, m] = sum of x[m]^2 over columns 16 b .. 16 b + 15.
+    whole_lines False (tests): the weights are loaded in operand layout also where whole cache lines would apply."""
     import ctypes
     _dev(a, w, out)
     M, K = a.shape
@@ -390,10 +452,16 @@ def gemm_nt(a, w, out, alpha: float = 1.0, swiglu_output: bool = False, row_fact
         _need(x.dtype == torch.float32 and tuple(x.shape) == (M, N) and x.stride(1) == 1, "gemm_nt: residual stream must be float32 [M, N]")
         _need(weight.dtype == torch.float32 and weight.is_contiguous() and weight.numel() == N, "gemm_nt: norm weight must be float32 [N]")
         _need(sumsq_out.dtype == torch.float32 and sumsq_out.is_contiguous()
-              and tuple(sumsq_out.shape) == (residual_parts(N), 16) and residual_parts(N) <= MAX_SUMSQ_PARTS,
+              and tuple(sumsq_out.shape) == (residual_parts(N), 16) and residual_parts(N) <= max_sumsq_parts(),
               "gemm_nt: sumsq_out must be float32 [residual_parts(N) <= 256, 16]")
         rn = IcResidualNorm(x.data_ptr(), x.stride(0), weight.data_ptr(), float(beta), sumsq_out.data_ptr(), sumsq_out.shape[0])
         mode = 2
+    if not whole_lines:
+        check(get_lib().ic_gemm_nt_variant(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
+                                           out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),
+                                           out.stride(0), float(alpha), mode, ctypes.byref(rf) if rf else None,
+                                           ctypes.byref(rn) if rn else None, 0, _stream()), "gemm_nt")
+        return out
     check(get_lib().ic_gemm_nt(a.data_ptr(), dtype_code(a.dtype), w.data_ptr(), dtype_code(w.dtype),
                                out.data_ptr(), dtype_code(out.dtype), M, N, K, a.stride(0), w.stride(0),
                                out.stride(0), float(alpha), mode, ctypes.byref(rf) if rf else None,
@@ -500,17 +568,12 @@ def gemm_qkv_rope_supported(dtype, head_dim: int) -> bool:
         return False
 
 
-def gemm_qkv_rope_tile_rows(rows: int) -> None:
-    """For tuning and tests: weight rows per tile that gemm_qkv_rope uses (16, 8 or 4; 0: chosen from the number
-    of heads, so that few heads still make a block for every compute unit)."""
-    check(get_lib().ic_gemm_qkv_rope_tile_rows(int(rows)), "gemm_qkv_rope_tile_rows")
-
-
 def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads, n_kv_heads, head_dim, page_size,
-                  row_factor=None):
+                  row_factor=None, tile_rows: int = 0):
     """For M <= gemm_epilogue_rows("rope", a, w) rows: qkv = a @ w^T with the rotary encoding and the cache write in the epilogue.
     The q heads of qkv[M, >= n_heads * head_dim] hold rotated queries afterwards; rotated keys and
-    the values are in cache slot ``slots[m]``.  Full rotary, bfloat16.  row_factor: as in gemm_nt."""
+    the values are in cache slot ``slots[m]``.  Full rotary, bfloat16.  row_factor: as in gemm_nt.
+    tile_rows (tests): used weight rows per tile, 16, 8 or 4; 0: chosen from the number of heads."""
     import ctypes
     _dev(a, w, qkv, positions, slots, cos, sin, kcache, vcache)
     M, K = a.shape
@@ -526,10 +589,13 @@ def gemm_qkv_rope(a, w, qkv, positions, slots, cos, sin, kcache, vcache, n_heads
           and cos.shape[-1] == head_dim // 2 and sin.shape == cos.shape, "gemm_qkv_rope: cos/sin must be float32 [max_pos, dh/2]")
     _need(kcache.is_contiguous() and vcache.is_contiguous() and kcache.shape == vcache.shape
           and tuple(kcache.shape[1:]) == (n_kv_heads, page_size, head_dim), "gemm_qkv_rope: cache layout")
-    check(get_lib().ic_gemm_qkv_rope(a.data_ptr(), w.data_ptr(), qkv.data_ptr(), M, K, a.stride(0), w.stride(0),
-                                     qkv.stride(0), positions.data_ptr(), slots.data_ptr(), cos.data_ptr(),
-                                     sin.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), n_heads, n_kv_heads,
-                                     head_dim, page_size, ctypes.byref(rf) if rf else None, _stream()), "gemm_qkv_rope")
+    args = (a.data_ptr(), w.data_ptr(), qkv.data_ptr(), M, K, a.stride(0), w.stride(0), qkv.stride(0), positions.data_ptr(),
+            slots.data_ptr(), cos.data_ptr(), sin.data_ptr(), kcache.data_ptr(), vcache.data_ptr(), n_heads, n_kv_heads,
+            head_dim, page_size, ctypes.byref(rf) if rf else None)
+    if tile_rows:
+        check(get_lib().ic_gemm_qkv_rope_variant(*args, int(tile_rows), _stream()), "gemm_qkv_rope")
+    else:
+        check(get_lib().ic_gemm_qkv_rope(*args, _stream()), "gemm_qkv_rope")
     return qkv
 
 

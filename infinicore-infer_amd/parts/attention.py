@@ -127,13 +127,12 @@ class Attention(Mixer):
     def _attend(self, q, out, ctx, cache):
         rt = self.runtime
         args = (self.nh, self.nkvh, self.dh, ctx.page_size)
-        fast = rt.attention_impl == "auto"
-        dec_ok = fast and ops.attention_decode_supported(rt.dtype, self.dh)
-        pre_ok = fast and ops.attention_prefill_supported(rt.dtype, self.dh, ctx.page_size)
         n_dec, n_tiles = ctx.n_decode_rows, ctx.n_prefill_tiles
-        use_dec = dec_ok and n_dec > 0 and (pre_ok or n_tiles == 0)
-        use_pre = pre_ok and n_tiles > 0 and (dec_ok or n_dec == 0)
-        if not ((use_dec or n_dec == 0) and (use_pre or n_tiles == 0)):
+        how = ops.ATTN_GENERAL
+        if rt.attention_impl == "auto":
+            how = ops.rule_attention(rt.dtype, self.dh, ctx.page_size, n_dec, n_tiles)
+        use_dec, use_pre = bool(how & ops.ATTN_SINGLE_TOKENS), bool(how & ops.ATTN_PORTIONS)
+        if how == ops.ATTN_GENERAL:
             ops.attention_generic(q, out, cache.k, cache.v, cache.block_tables, ctx.token_req, ctx.positions,
                                   *args, self.scale, self.window)
             return
@@ -151,9 +150,11 @@ class Attention(Mixer):
             if self.window:
                 keys = min(keys, self.window + ops.attention_prefill_tile_rows())
             parts, part_len = ops.attention_prefill_parts(n_tiles, self.nh, self.dh, keys, ctx.cu_count)
-            scratch = None
+            scratch = counters = None
             if parts > 1:
                 scratch = ctx.ws.buffer("attn_tile_parts", (ops.attention_prefill_scratch_floats(n_tiles, self.nh, self.dh, parts),),
                                         torch.float32)
+                counters = ctx.ws.zeroed("attn_tile_arrivals", (ops.attention_prefill_counter_ints(),), torch.int32)
             ops.attention_prefill(q, out, cache.k, cache.v, cache.block_tables, ctx.prefill_tiles, n_tiles,
-                                  *args, self.scale, self.window, parts=parts, part_len=part_len, scratch=scratch)
+                                  *args, self.scale, self.window, parts=parts, part_len=part_len, scratch=scratch,
+                                  counters=counters)

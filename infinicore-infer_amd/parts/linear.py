@@ -16,8 +16,9 @@ from .base import DeferredRows
 torch.backends.cuda.matmul.allow_tf32 = False
 torch.backends.cudnn.allow_tf32 = False
 
-FEW_ROWS = 16          # up to here the package's own kernel beats the library on MI355X
-MID_ROWS = 64          # up to here the sliced product beats it for results as wide as the model (O, down)
+# Which product runs where (own kernel up to some rows, slices over K for the projections into the residual
+# stream, the library beyond) is the kernel library's rule, asked through ops.rule_*: its native step function
+# asks the same functions, so the two ways of issuing a step choose alike.
 TUNE_LIBRARY = False   # while True, every library product times the library's algorithms for its shape first
 TUNE_FLUSH = None      # while tuning: a tensor larger than the caches, overwritten before every timed launch
 _tuned = set()
@@ -46,8 +47,7 @@ def _library(x, w, out, alpha: float = 1.0):
 
 
 def own_kernel_applies(M, x_dtype, w_dtype, out_dtype, impl: str) -> bool:
-    return (impl == "auto" and M <= FEW_ROWS and x_dtype == torch.bfloat16 and w_dtype == torch.bfloat16
-            and ops.gemm_nt_supported(x_dtype, w_dtype, out_dtype))
+    return impl == "auto" and ops.rule_own_product(x_dtype, w_dtype, out_dtype, M)
 
 
 def linear(x, w, out, impl: str = "auto", alpha: float = 1.0):
@@ -76,10 +76,12 @@ def linear_tail(x, w, tail, ws, name: str, impl: str = "auto"):
     epilogue: returns ``DeferredRows`` for that norm, or None when this step cannot be done so
     (many rows, float32, a width beyond the kernel's) and the caller computes the plain product."""
     M, N = x.shape[0], w.shape[0]
-    if tail is None:
+    if tail is None or impl != "auto" or tuple(tail.x.shape) != (M, N) or x.stride(1) != 1 or w.stride(1) != 1:
         return None
-    if (impl == "auto" and M <= MID_ROWS and tuple(tail.x.shape) == (M, N) and N % 4 == 0
-            and ops.gemm_splitk_supported(x, w) and ops.gemm_splitk_pays(M, N, w.shape[1])):
+    how = ops.rule_tail(x.dtype, x, w)
+    if how == ops.TAIL_PLAIN:
+        return None
+    if how == ops.TAIL_SLICES:
         # 17..64 rows into the residual stream (and 13..16 long ones): the product as slices over K; the kernel that
         # sums them does the add and the whole norm, so the rows handed on owe nothing
         slices = ops.gemm_splitk_slices(N, w.shape[1])
@@ -87,11 +89,7 @@ def linear_tail(x, w, tail, ws, name: str, impl: str = "auto"):
         y = ws.buffer(name + "_values", (M, N), torch.bfloat16)
         ops.splitk_add_rmsnorm(parts, tail.x, tail.alpha, tail.weight, y, tail.eps)
         return DeferredRows(y, None, N, tail.eps)
-    if not own_kernel_applies(M, x.dtype, w.dtype, torch.bfloat16, impl):
-        return None
     parts = ops.residual_parts(N)
-    if parts > ops.MAX_SUMSQ_PARTS or tuple(tail.x.shape) != (M, N):
-        return None
     y = ws.buffer(name + "_values", (M, N), torch.bfloat16)
     sumsq = ws.buffer(name + "_sumsq", (parts, 16), torch.float32)
     ops.gemm_nt(x, w, y, residual=(tail.x, tail.weight, tail.alpha, sumsq))

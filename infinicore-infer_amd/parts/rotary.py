@@ -19,7 +19,6 @@ import torch
 
 from ..kernels import ops
 from .base import DeferredRows, PositionEncoding, register_part
-from .linear import FEW_ROWS
 
 
 def rotary_tables(head_dim, theta, max_positions, scaling=None, rot_dim=None, model_max_positions=None):
@@ -93,12 +92,9 @@ class Rotary(PositionEncoding):
         row_factor = None
         if isinstance(h, DeferredRows):
             h, row_factor = h.values, h.row_factor()
-        if (rt.gemm_impl != "auto" or n_kv_heads == 0 or self.rot_dim != head_dim
-                or h.dtype != torch.bfloat16 or w_qkv.dtype != torch.bfloat16
-                or not ops.gemm_qkv_rope_supported(h.dtype, head_dim)):
-            return False
-        # up to 16 rows, or as many as the kernel takes with whole-line weight loads when no row factors are owed
-        if h.shape[0] > FEW_ROWS and (row_factor is not None or h.shape[0] > ops.gemm_epilogue_rows("rope", h, w_qkv)):
+        if (rt.gemm_impl != "auto" or h.dtype != w_qkv.dtype or h.dtype != qkv.dtype
+                or not ops.rule_qkv_fused(h.dtype, h.shape[0], h, w_qkv, head_dim, self.rot_dim, n_kv_heads,
+                                          row_factor is not None)):
             return False
         if ctx.max_position >= self.max_positions:
             raise ValueError("position %d is beyond the rotary tables (%d)" % (ctx.max_position, self.max_positions))

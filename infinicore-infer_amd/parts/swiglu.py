@@ -10,7 +10,7 @@ import torch
 from ..kernels import ops
 from ..weights.loader import WeightSpec
 from .base import DeferredRows, FeedForward, register_part
-from .linear import linear, linear_tail, own_kernel_applies
+from .linear import linear, linear_tail
 
 
 @register_part("feed_forward", "swiglu")
@@ -56,11 +56,14 @@ class SwiGLU(FeedForward):
 
     def forward(self, h, ctx, tail=None):
         rt = self.runtime
+        if isinstance(h, DeferredRows) and h.sumsq is None:
+            h = h.values                   # the whole norm is applied already: plain rows, nothing owed
         T = h.shape[0]
         act = ctx.ws.buffer("ffn_act", (T, self.intermediate_size), rt.dtype)
-        few = own_kernel_applies(T, h.dtype, self.w_gate_up.dtype, act.dtype, rt.gemm_impl)
-        if not few and not isinstance(h, DeferredRows) and own_kernel_applies(1, h.dtype, self.w_gate_up.dtype, act.dtype, rt.gemm_impl):
-            few = T <= ops.gemm_epilogue_rows("swiglu", h, self.w_gate_up)      # up to 32 rows with whole-line weight loads
+        owed = isinstance(h, DeferredRows)
+        rows = h.values if owed else h
+        few = (rt.gemm_impl == "auto" and rows.dtype == self.w_gate_up.dtype == act.dtype
+               and ops.rule_gate_up_fused(rows.dtype, T, rows, self.w_gate_up, owed))
         if few:
             # few rows: the activation is the epilogue of the gate/up projection
             if isinstance(h, DeferredRows):

@@ -100,9 +100,10 @@ def random_state_dict(config: dict, seed: int, std: float = 0.02, norm_std: floa
     if tie is None:
         tie = config.get("tie_word_embeddings", True)
     out: Dict[str, torch.Tensor] = {}
-    for name, spec in model.weight_specs().items():
-        if tie and name == "lm_head.weight":
-            continue
+    specs = model.weight_specs()
+    for name, spec in specs.items():
+        if tie and spec.fallback in specs and spec.fallback in out:
+            continue                # a tied tensor is not written: the loader takes the tensor it falls back to
         t = _draw(seed, name, spec.shape, spec.role, std, norm_std, device)
         out[name] = (t if spec.role == "vector" else t.to(dtype)).contiguous()
     return out

@@ -159,15 +159,34 @@ def trace_mixed(requests, live_max=4, sizes=(7, 2, 16, 3, 11, 2, 29, 5), tail=6,
     return steps, peak
 
 
+def wanted_places(steps):
+    """The set of (id, position) whose logits a trace asks for."""
+    places, cursor = set(), {}
+    for rec in steps:
+        for e in rec["entries"]:
+            base = cursor.get(e["id"], 0)
+            places.update((e["id"], base + w) for w in e["want"])
+            cursor[e["id"]] = base + len(e["tokens"])
+        for rid in rec["end"]:
+            cursor.pop(rid, None)
+    return places
+
+
 def run_trace(engine, steps):
-    """Feed steps to the engine; returns {(id, position): float32 logits row (CPU)}."""
+    """Feed steps to the engine; returns {(id, position): float32 logits row (CPU)}.  A step must return exactly
+    one row for every place it wants: a step that returns nothing, or too few rows, fails here."""
     from infinicore_infer_amd.engine import StepEntry
     got = {}
     cursor = {}
     for rec in steps:
         entries = [StepEntry(e["id"], e["tokens"], e["want"]) for e in rec["entries"]]
         logits = engine.step(entries)
-        if logits is not None:
+        n_wanted = sum(len(e["want"]) for e in rec["entries"])
+        if n_wanted == 0:
+            assert logits is None, "step %s wants nothing and got logits" % rec.get("step")
+        else:
+            assert logits is not None, "step %s wants %d rows and got none" % (rec.get("step"), n_wanted)
+            assert logits.shape[0] == n_wanted, "step %s wants %d rows and got %d" % (rec.get("step"), n_wanted, logits.shape[0])
             rows = logits.float().cpu()
             i = 0
             for e in rec["entries"]:
@@ -175,7 +194,6 @@ def run_trace(engine, steps):
                 for w in e["want"]:
                     got[(e["id"], base + w)] = rows[i].clone()
                     i += 1
-            assert i == rows.shape[0]
         for e in rec["entries"]:
             cursor[e["id"]] = cursor.get(e["id"], 0) + len(e["tokens"])
         for rid in rec["end"]:
@@ -190,8 +208,14 @@ def plain_logits(cfg, sd, requests, bf16):
             for rid, toks in requests.items()}
 
 
-def compare(got, ref, tol, what=""):
-    """Every wanted row against the plain logits; reports the first wrong place."""
+def compare(got, ref, tol, what="", steps=None):
+    """Every wanted row against the plain logits; reports the first wrong place.  ``got`` must hold rows (with
+    ``steps`` given: exactly the places the trace wants), so a run that returned nothing cannot pass."""
+    assert len(got) > 0, "%s: no logits to compare" % what
+    if steps is not None:
+        want = wanted_places(steps)
+        assert set(got) == want, ("%s: %d of %d wanted places came back (missing e.g. %s)"
+                                  % (what, len(set(got) & want), len(want), sorted(want - set(got), key=str)[:3]))
     worst, worst_at = 0.0, None
     for (rid, pos), row in sorted(got.items(), key=lambda kv: (str(kv[0][0]), kv[0][1])):
         r = ref[rid][pos]

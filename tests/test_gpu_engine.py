@@ -164,6 +164,47 @@ def test_fourteen_rows_of_16_kb_go_through_the_sliced_product(tmp_path_factory, 
     engine.cache.check_invariants()
 
 
+@pytest.mark.parametrize("n_req", [20, 40])
+def test_seventeen_to_sixty_four_rows_at_a_width_where_the_slices_pay(tmp_path_factory, n_req):
+    """20 and 40 requests decode together on a model wide enough that its O and down projections run as slices over
+    K (hidden 1,024, inner size 8,192): sliced O with the whole norm applied, the gate/up product fed fully normed rows
+    (with the SwiGLU epilogue at 20 rows, the library's product and the activation kernel at 40), sliced down, and the
+    head fed normed rows.  The logits equal the plain model's, and the step issued by native code and the one issued
+    by the parts' Python forward launch the same kernels: their logits are equal to the bit."""
+    from infinicore_infer_amd.engine import Engine, StepEntry
+    from infinicore_infer_amd.kernels import ops
+    from infinicore_infer_amd.weights import write_random_model
+    import os
+    cfg = dict(model_type="minicpm", vocab_size=1003, hidden_size=1024, num_hidden_layers=2, num_attention_heads=8,
+               num_key_value_heads=2, intermediate_size=8192, max_position_embeddings=256, rms_norm_eps=1e-5,
+               rope_theta=10000.0, scale_emb=4, dim_model_base=256, scale_depth=1.4, tie_word_embeddings=False, eos_token_id=2)
+    assert ops.gemm_splitk_pays(n_req, 1024, 8192) and ops.gemm_splitk_pays(n_req, 1024, 1024)
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "model_long_rows")
+    if not os.path.exists(os.path.join(folder, "model.safetensors")):
+        write_random_model(folder, cfg, seed=21, std=0.02)
+    n_dec = 3
+    lens = [2 + (5 * i) % 23 for i in range(n_req)]
+    requests = {"s%d" % i: H.random_tokens(cfg["vocab_size"], lens[i] + n_dec, 900 + i) for i in range(n_req)}
+    steps = [{"step": 0, "end": [],
+              "entries": [{"id": k, "tokens": t[:lens[i]], "want": [lens[i] - 1]} for i, (k, t) in enumerate(requests.items())]}]
+    for j in range(n_dec):
+        steps.append({"step": j + 1, "end": list(requests) if j == n_dec - 1 else [],
+                      "entries": [{"id": k, "tokens": [t[lens[i] + j]], "want": [0]} for i, (k, t) in enumerate(requests.items())]})
+    ref = H.plain_logits(cfg, H.load_state_dict(folder), requests, True)
+    got = {}
+    for native in (True, False):
+        engine = Engine.from_dir(folder, dtype=torch.bfloat16, max_tokens=n_req * 64, page_size=16, max_requests=n_req,
+                                 use_native=native, use_graphs=False)
+        assert (engine.native is not None) == native
+        got[native] = H.run_trace(engine, steps)
+        assert len(got[native]) == n_req * (1 + n_dec)
+        H.compare(got[native], ref, H.BF16_TOL, "%d requests at width 1,024, native %s" % (n_req, native), steps=steps)
+        engine.cache.check_invariants()
+    assert set(got[True]) == set(got[False])
+    for key in got[True]:
+        assert torch.equal(got[True][key], got[False][key]), "native and Python-issued steps differ at %r" % (key,)
+
+
 def test_out_of_pages_changes_nothing(tmp_path_factory):
     from infinicore_infer_amd.cache import OutOfPages
     from infinicore_infer_amd.engine import StepEntry

@@ -208,10 +208,12 @@ def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_w
         tl = torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 4)
         if parts:
             scratch = torch.full((ops.attention_prefill_scratch_floats(tl.shape[0], nh, dh, parts[0]),), float("nan"), device=DEV)
+            counters = torch.zeros(ops.attention_prefill_counter_ints(), dtype=torch.int32, device=DEV)
             for _ in range(2):
                 out.zero_()
                 ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0, 1,
-                                      parts=parts[0], part_len=parts[1], scratch=scratch)
+                                      parts=parts[0], part_len=parts[1], scratch=scratch, counters=counters)
+                assert int(counters.abs().sum()) == 0          # every launch leaves its arrival counters at zero
         else:
             ops.attention_prefill(q, out, kc, vc, btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, window or 0, groups)
     return out, torch.cat(want)
@@ -272,10 +274,15 @@ def test_attention_prefill_parts_rule_and_its_refusals():
     bt = torch.zeros(1, 2, dtype=torch.int32, device=DEV)
     tl = torch.tensor([[0, 0, 128, 0]], dtype=torch.int32, device=DEV)
     small = torch.zeros(16, device=DEV)
+    counters = torch.zeros(ops.attention_prefill_counter_ints(), dtype=torch.int32, device=DEV)
     with pytest.raises(ops.KernelError):        # scratch memory too small for two parts
-        ops.attention_prefill(q, torch.zeros_like(q), kc, kc, bt, tl, 1, 1, 1, 64, 64, 0.125, 0, 1, parts=2, part_len=1, scratch=small)
+        ops.attention_prefill(q, torch.zeros_like(q), kc, kc, bt, tl, 1, 1, 1, 64, 64, 0.125, 0, 1, parts=2, part_len=1, scratch=small,
+                              counters=counters)
     with pytest.raises(ops.KernelError):        # parts go with one wave group only
         ops.attention_prefill(q, torch.zeros_like(q), kc, kc, bt, tl, 1, 1, 1, 64, 64, 0.125, 0, 2, parts=2, part_len=1,
+                              scratch=torch.zeros(2 * 256 * 34, device=DEV), counters=counters)
+    with pytest.raises(ops.KernelError):        # a cut walk without arrival counters of the caller's
+        ops.attention_prefill(q, torch.zeros_like(q), kc, kc, bt, tl, 1, 1, 1, 64, 64, 0.125, 0, 1, parts=2, part_len=1,
                               scratch=torch.zeros(2 * 256 * 34, device=DEV))
 
 
@@ -552,7 +559,6 @@ def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page, tile_rows):
     rotary/cache-write kernel, with every number of used rows per tile (0: chosen from the heads)."""
     g = torch.Generator().manual_seed(31)
     ops = _ops()
-    ops.gemm_qkv_rope_tile_rows(tile_rows)
     H = (nh + 2 * nkvh) * dh
     h = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (torch.randn(H, K, generator=g) * 0.1).to(torch.bfloat16)
@@ -566,10 +572,8 @@ def test_gemm_qkv_rope(M, nh, nkvh, dh, K, page, tile_rows):
     kc = torch.zeros(n_pages, nkvh, page, dh, dtype=torch.bfloat16, device=DEV)
     vc = torch.zeros_like(kc)
     qkv = torch.zeros(M, H, dtype=torch.bfloat16, device=DEV)
-    try:
-        ops.gemm_qkv_rope(h.to(DEV), w.to(DEV), qkv, pos.to(DEV), slots.to(DEV), cos, sin, kc, vc, nh, nkvh, dh, page)
-    finally:
-        ops.gemm_qkv_rope_tile_rows(0)
+    ops.gemm_qkv_rope(h.to(DEV), w.to(DEV), qkv, pos.to(DEV), slots.to(DEV), cos, sin, kc, vc, nh, nkvh, dh, page,
+                      tile_rows=tile_rows)
     # the two-kernel path
     kc2, vc2 = torch.zeros_like(kc), torch.zeros_like(vc)
     ref = torch.empty(M, H, dtype=torch.bfloat16, device=DEV)
@@ -636,21 +640,16 @@ def test_the_head_product_with_whole_line_weight_loads(M, N, K, out_dtype):
     """Very many weight rows (the output head): from rows of 4 KB that are whole cache lines the kernel whose waves own
     whole weight tiles reads them line by line through LDS; switched off it loads in operand layout.  The two add the same
     products in the same order, so they agree to the bit, and both give the plain product."""
-    from infinicore_infer_amd.kernels.lib import get_lib
-    ops, lib = _ops(), get_lib()
+    ops = _ops()
     g = torch.Generator().manual_seed(67)
     a = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16)
     ad, wd = a.to(DEV), w.to(DEV)
     got = {}
-    try:
-        for on in (1, 0):
-            lib.ic_gemm_nt_lines_enable(on)
-            out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
-            ops.gemm_nt(ad, wd, out, 0.25)
-            got[on] = out.cpu()
-    finally:
-        lib.ic_gemm_nt_lines_enable(1)
+    for on in (1, 0):
+        out = torch.full((M, N), float("nan"), dtype=out_dtype, device=DEV)
+        ops.gemm_nt(ad, wd, out, 0.25, whole_lines=bool(on))
+        got[on] = out.cpu()
     assert torch.equal(got[1], got[0])
     _close(got[1], 0.25 * P.plain_linear(a, w), out_dtype, factor=20 if out_dtype == torch.float32 else 2)
 
@@ -661,8 +660,7 @@ def test_whole_line_weight_loads_equal_loads_in_operand_layout(M, N, K):
     """With K a multiple of 64 the few-row products read their weights in whole cache lines and pass them through LDS;
     switched off, the same entry points load in operand layout.  Both must give the plain product, the activation
     epilogue and the residual epilogue alike (rows of 16 KB and more: a wave owns a run of k-steps)."""
-    from infinicore_infer_amd.kernels.lib import get_lib
-    ops, lib = _ops(), get_lib()
+    ops = _ops()
     g = torch.Generator().manual_seed(61)
     a = torch.randn(M, K, generator=g).to(torch.bfloat16)
     w = (torch.randn(N, K, generator=g) * 0.1).to(torch.bfloat16)
@@ -670,24 +668,21 @@ def test_whole_line_weight_loads_equal_loads_in_operand_layout(M, N, K):
     gw = torch.rand(N, generator=g) + 0.5
     ad, wd = a.to(DEV), w.to(DEV)
     got = {}
-    try:
-        for on in (1, 0):
-            lib.ic_gemm_nt_lines_enable(on)
-            plain = torch.empty(M, N, dtype=torch.float32, device=DEV)
-            ops.gemm_nt(ad, wd, plain, 0.5)
-            res = None
-            if N % 2 == 0:
-                act = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
-                ops.gemm_nt(ad, wd, act, swiglu_output=True)
-                xd = x.to(DEV)
-                y = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
-                if ops.residual_parts(N) <= ops.MAX_SUMSQ_PARTS:
-                    sumsq = torch.zeros(ops.residual_parts(N), 16, device=DEV)
-                    ops.gemm_nt(ad, wd, y, residual=(xd, gw.to(DEV), 0.3, sumsq))
-                res = (act.float().cpu(), xd.cpu(), y.float().cpu())
-            got[on] = (plain.cpu(), res)
-    finally:
-        lib.ic_gemm_nt_lines_enable(1)
+    for on in (1, 0):
+        lines = bool(on)
+        plain = torch.empty(M, N, dtype=torch.float32, device=DEV)
+        ops.gemm_nt(ad, wd, plain, 0.5, whole_lines=lines)
+        res = None
+        if N % 2 == 0:
+            act = torch.empty(M, N // 2, dtype=torch.bfloat16, device=DEV)
+            ops.gemm_nt(ad, wd, act, swiglu_output=True, whole_lines=lines)
+            xd = x.to(DEV)
+            y = torch.zeros(M, N, dtype=torch.bfloat16, device=DEV)
+            if ops.residual_parts(N) <= ops.max_sumsq_parts():
+                sumsq = torch.zeros(ops.residual_parts(N), 16, device=DEV)
+                ops.gemm_nt(ad, wd, y, residual=(xd, gw.to(DEV), 0.3, sumsq), whole_lines=lines)
+            res = (act.float().cpu(), xd.cpu(), y.float().cpu())
+        got[on] = (plain.cpu(), res)
     want = 0.5 * P.plain_linear(a, w)
     for on in (1, 0):
         _close(got[on][0], want, torch.float32, factor=20)
@@ -696,7 +691,7 @@ def test_whole_line_weight_loads_equal_loads_in_operand_layout(M, N, K):
         for on in (1, 0):
             act, xs, y = got[on][1]
             _close(act, P.plain_swiglu(gu[:, :N // 2], gu[:, N // 2:]), torch.bfloat16, factor=2)
-            if ops.residual_parts(N) <= ops.MAX_SUMSQ_PARTS:
+            if ops.residual_parts(N) <= ops.max_sumsq_parts():
                 _close(xs, x.double() + 0.3 * gu, torch.bfloat16, scale=0.3 * float(gu.abs().max()))
                 _close(y, xs.double() * gw.double(), torch.bfloat16)
 

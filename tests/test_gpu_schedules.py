@@ -462,3 +462,72 @@ def test_prefix_cache_through_the_entry_point(tmp_path, name):
     model._scheduler.release_idle()
     model.engine.cache.check_invariants()
     assert model.engine.cache.free_pages(0) == model.engine.num_pages
+
+
+# ---- the reference's own generation loop over the Python surface -----------------------------------------------------------
+@pytest.mark.parametrize("dname", ["float32", "bfloat16"])
+@pytest.mark.parametrize("name", ["A", "B"])
+def test_the_reference_loop_over_the_python_surface(tmp_path, name, dname):
+    """Generation written as the reference writes it (scripts/jiuge.py:548-586): create_kv_cache, InferTask.bind_kvcache,
+    batch_infer_one_round, task.next, drop_kv_cache.  Two tasks step together, as the reference's server batches them
+    (scripts/launch_server.py:134-159); a third starts from a duplicated cache (duplicateKVCache, jiuge.h:66-69) and
+    must go on exactly as the task it was copied from.  All against the plain implementation."""
+    from plain_model import plain_generate, round_bf16
+    from infinicore_infer_amd.engine.tasks import InferTask
+    from infinicore_infer_amd.minicpm import MiniCPMForCausalLM
+    folder = H.make_model_dir(tmp_path, name, seed=8)
+    cfg = H.CONFIGS[name][0]
+    sd = H.load_state_dict(folder)
+    rnd = round_bf16 if dname == "bfloat16" else None
+    model = MiniCPMForCausalLM(folder, dtype=getattr(torch, dname), cache_tokens=1024, page_size=16, max_requests=8)
+    assert model.max_context_len() == cfg["max_position_embeddings"]
+    n_new = 9
+    prompts = [H.random_tokens(cfg["vocab_size"], n, 60 + i) for i, n in enumerate([11, 30])]
+    tasks = []
+    for i, p in enumerate(prompts):
+        t = InferTask(i, p, model.max_context_len(), 1.0, 1, 1.0, [])       # topk 1: greedy, the reference's default
+        t.bind_kvcache(model.create_kv_cache())
+        tasks.append(t)
+    outs = [[] for _ in tasks]
+    fork_at, forked, forked_out = 4, None, []
+    for step in range(n_new):
+        out = model.batch_infer_one_round(tasks)
+        assert len(out) == len(tasks)
+        for i, (t, tok) in enumerate(zip(tasks, out)):
+            outs[i].append(int(tok))
+            t.next(int(tok))
+            assert t.kvcache().tokens == (prompts[i] + outs[i])[:t.pos] and t.finish_reason is None
+        if step == fork_at:
+            # a second cache with a copy of what task 0's cache holds now; a new task goes on from there
+            src = tasks[0]
+            copy = model.duplicate_kv_cache(src.kvcache(), src.pos)
+            assert copy.tokens == src.kvcache().tokens and copy.data() != src.kvcache().data()
+            forked = InferTask("fork", prompts[0] + outs[0], model.max_context_len(), 1.0, 1, 1.0, [])
+            forked.bind_kvcache(copy, src.pos)                         # only the token after the copied ones is left to feed
+            assert forked.tokens == [outs[0][-1]]
+    for step in range(n_new - fork_at - 1):
+        tok = int(model.batch_infer_one_round([forked])[0])
+        forked_out.append(tok)
+        forked.next(tok)
+    for i, p in enumerate(prompts):
+        assert outs[i] == plain_generate(cfg, sd, p, n_new, rnd=rnd), "task %d" % i
+    assert forked_out == outs[0][fork_at + 1:]
+    # the finish rules of scripts/infer_task.py:27-36: an end token stops, the position limit ends by length
+    t = InferTask("e", prompts[0], model.max_context_len(), 1.0, 1, 1.0, [outs[0][2]])
+    t.bind_kvcache(model.create_kv_cache())
+    for j in range(outs[0].index(outs[0][2]) + 1):
+        assert t.finish_reason is None
+        t.next(int(model.batch_infer_one_round([t])[0]))
+    assert t.finish_reason == "stop" and t.generated == outs[0][:outs[0].index(outs[0][2]) + 1]
+    t2 = InferTask("l", prompts[0], len(prompts[0]) + 1, 1.0, 1, 1.0, [])
+    t2.bind_kvcache(model.create_kv_cache())
+    t2.next(int(model.batch_infer_one_round([t2])[0]))
+    assert t2.finish_reason is None
+    t2.next(int(model.batch_infer_one_round([t2])[0]))
+    assert t2.finish_reason == "length"
+    for task in tasks + [forked, t, t2]:
+        model.drop_kv_cache(task.release_kvcache())
+        assert task.kvcache() is None
+    model.engine.cache.check_invariants()
+    assert all(model.engine.cache.free_pages(g) == model.engine.cache.pools[g].num_pages for g in range(len(model.engine.groups)))
+    model.destroy_model_instance()

@@ -391,3 +391,32 @@ def test_decoding_ahead_issues_the_next_step_before_it_reads_the_tokens():
     # without the two calls, or with kept caches, the scheduler stays as it was
     assert not Scheduler(FakeEngine(8), overlap=True).overlap
     assert not Scheduler(AheadEngine(8), overlap=True, prefix_cache=True).overlap
+
+
+def test_more_running_requests_than_the_engine_runs_ahead():
+    """An engine records decode steps up to ``graph_max_batch`` rows and its ``sample_ahead`` has buffers for as
+    many: with more running requests the scheduler must not ask it to run ahead (the step before has already
+    grown every cache, so a refusal there would lose its tokens)."""
+    class Capped(AheadEngine):
+        graph_max_batch = 2
+
+        def sample_ahead(self, logits, *a, **kw):
+            assert len(list(logits)) <= self.graph_max_batch, "asked to run ahead with more rows than it takes"
+            return super().sample_ahead(logits, *a, **kw)
+
+    def run(n_requests, overlap):
+        eng = Capped(64, max_requests=4)
+        s = Scheduler(eng, max_batch_tokens=64, chunk_size=64, overlap=overlap)
+        for i in range(n_requests):
+            s.add(_task("q%d" % i, [1 + i, 2, 3], (4, 14, 15)[i]))
+        done = s.run()
+        eng.cache.check_invariants()
+        return {t.id: t.generated for t in done}, s
+
+    three, s3 = run(3, True)
+    assert three == run(3, False)[0] and len(three) == 3
+    assert [len(three["q%d" % i]) for i in range(3)] == [4, 14, 15]
+    # three rows never ran ahead; once one request has ended, the two that are left do
+    assert 0 < s3.n_ahead <= 10
+    two, s2 = run(2, True)
+    assert two == run(2, False)[0] and s2.n_ahead >= 8
