@@ -725,7 +725,7 @@ def test_gemm_qkv_rope_with_row_factors():
 
 # ---------------------------------------------------------------------------
 @pytest.mark.parametrize("M,N,K,S", [(1, 64, 128, 1), (17, 2304, 2304, 0), (33, 200, 344, 1), (64, 2304, 5760, 0), (48, 1000, 1096, 2),
-                                      (64, 331, 8, 1), (20, 4096, 8192, 0), (64, 136, 520, 1), (31, 777, 1160, 3)])
+                                      (64, 331, 64, 1), (5, 77, 72, 1), (20, 4096, 8192, 0), (64, 136, 520, 1), (31, 777, 1160, 3)])
 def test_gemm_in_slices_and_the_add_norm_that_sums_them(M, N, K, S):
     """The product of 1..64 rows as float32 slices over K (sizes that are no multiple of the block's 64 columns
     or of its chunk of 128 k; slices of unequal length), against float64; then the kernel that sums the slices,
@@ -735,6 +735,9 @@ def test_gemm_in_slices_and_the_add_norm_that_sums_them(M, N, K, S):
     a = torch.randn(M, K, generator=g).to(torch.bfloat16).to(DEV)
     w = (torch.randn(N, K, generator=g) / math.sqrt(K)).to(torch.bfloat16).to(DEV)
     assert ops.gemm_splitk_supported(a, w)
+    # rows shorter than 64 elements are refused (a clamped load of the last chunk would read past the row's end)
+    assert not ops.gemm_splitk_supported(a[:, :8].contiguous(), w[:, :8].contiguous())
+    assert not ops.gemm_splitk_supported(a[:, :56].contiguous(), w[:, :56].contiguous())
     slices = S or ops.gemm_splitk_slices(N, K)
     parts = torch.full((slices * M * N + 64,), float("nan"), device=DEV)
     p = ops.gemm_splitk(a, w, parts, slices)
