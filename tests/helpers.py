@@ -227,3 +227,23 @@ def compare(got, ref, tol, what="", steps=None):
         assert err <= tol, ("%s: request %s position %d differs by %.3g of the largest logit (allowed %.3g)"
                             % (what, rid, pos, err, tol))
     return worst, worst_at
+
+
+def compare_places(got, ref, tol, what=""):
+    """As ``compare`` for runs where only some positions were computed: ``ref`` maps (id, position) to the plain
+    logits row.  Every place of ``ref`` must be in ``got`` and nothing else; the error is taken as a fraction of the
+    largest plain logit of the request's rows."""
+    assert len(got) > 0 and set(got) == set(ref), ("%s: wanted %d places, got %d (missing e.g. %s)"
+                                                   % (what, len(ref), len(got), sorted(set(ref) - set(got), key=str)[:3]))
+    scale = {}
+    for (rid, _), r in ref.items():
+        scale[rid] = max(scale.get(rid, 0.0), float(r.abs().max()))
+    worst, worst_at = 0.0, None
+    for key in sorted(got, key=lambda k: (str(k[0]), k[1])):
+        err = float((got[key].double() - ref[key].double().cpu()).abs().max()) / scale[key[0]]
+        assert math.isfinite(err), "%s: non-finite logits at request %s position %d" % (what, key[0], key[1])
+        if err > worst:
+            worst, worst_at = err, key
+        assert err <= tol, ("%s: request %s position %d differs by %.3g of the largest logit (allowed %.3g)"
+                            % (what, key[0], key[1], err, tol))
+    return worst, worst_at

@@ -55,7 +55,7 @@ def plain_dims(cfg):
 def plain_embedding(table, tokens, scale):
     """x_i = E[token_i] * scale_emb.  jiuge.py:193-197 folds the scale into the
     table; src/models/jiuge/jiuge.cpp:164-168 copies one row per token."""
-    return table.to(F64)[torch.as_tensor(tokens, dtype=torch.long)] * scale
+    return table[torch.as_tensor(tokens, dtype=torch.long, device=table.device)].to(F64) * scale
 
 
 def plain_rmsnorm(x, w, eps):
@@ -73,7 +73,7 @@ def plain_linear(x, w):
     return x.to(F64) @ w.to(F64).t()
 
 
-def plain_rope_tables(dh, theta, npos, factors=None, magnitude=1.0):
+def plain_rope_tables(dh, theta, npos, factors=None, magnitude=1.0, device=None):
     """sin/cos[p, j] of angle p / theta^(j / (dh/2)), j < dh/2
     (src/models/jiuge/jiuge_weight.hpp:134-159, 161-186).  ``factors`` divides
     each pair's frequency and ``magnitude`` multiplies sin and cos (long-context
@@ -84,7 +84,7 @@ def plain_rope_tables(dh, theta, npos, factors=None, magnitude=1.0):
     if factors is not None:
         inv = inv / torch.as_tensor(factors, dtype=F64)
     ang = torch.arange(npos, dtype=F64)[:, None] * inv[None, :]
-    return torch.sin(ang) * magnitude, torch.cos(ang) * magnitude
+    return (torch.sin(ang) * magnitude).to(device), (torch.cos(ang) * magnitude).to(device)
 
 
 def plain_longrope(cfg):
@@ -113,7 +113,7 @@ def plain_rope_adjacent(x, positions, sin, cos):
     """Rotate adjacent pairs (2j, 2j+1) of every head by the angle of the token's
     position: (a, b) -> (a cos - b sin, a sin + b cos).  x: [T, n, dh].  Call
     sites jiuge.cpp:202-203."""
-    pos = torch.as_tensor(positions, dtype=torch.long)
+    pos = torch.as_tensor(positions, dtype=torch.long, device=x.device)
     s = sin[pos][:, None, :]
     c = cos[pos][:, None, :]
     a = x[..., 0::2]
@@ -134,9 +134,9 @@ def plain_attention(q, k, v, scale, past=0, window=None):
     s, nh, dh = q.shape
     t, nkvh, _ = k.shape
     g = nh // nkvh
-    out = torch.empty(s, nh, dh, dtype=F64)
-    qi = past + torch.arange(s)[:, None]
-    kj = torch.arange(t)[None, :]
+    out = torch.empty(s, nh, dh, dtype=F64, device=q.device)
+    qi = past + torch.arange(s, device=q.device)[:, None]
+    kj = torch.arange(t, device=q.device)[None, :]
     allowed = kj <= qi
     if window is not None:
         allowed = allowed & (kj > qi - window)
@@ -163,7 +163,9 @@ def plain_swiglu(gate, up):
 def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", window=None, start_pos=0,
                   rows=None):
     """Logits [T, vocab] (float64) of one request's whole token sequence from
-    position 0.  ``weights``: tensors by checkpoint name (jiuge.py:33-77)."""
+    position 0.  ``weights``: tensors by checkpoint name (jiuge.py:33-77); the
+    arithmetic runs where they lie (the large shapes are checked with the weights
+    on the GPU: the same float64 torch operations, only faster)."""
     rnd = rnd or _ident
     nh, nkvh, dh = plain_dims(cfg)
     L = cfg["num_hidden_layers"]
@@ -173,12 +175,11 @@ def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", 
     T = len(tokens)
     positions = list(range(start_pos, start_pos + T))     # start_pos != 0 only to test that distances alone count
     factors, magnitude = plain_longrope(cfg)
-    sin, cos = plain_rope_tables(dh, theta, start_pos + T, factors, magnitude)
-
     emb_name = "model.embed_tokens.weight"
     head_name = "lm_head.weight"
     emb = weights[emb_name] if emb_name in weights else weights[head_name]      # jiuge.py:182-186
     head = weights[head_name] if head_name in weights else weights[emb_name]    # jiuge.py:187-191
+    sin, cos = plain_rope_tables(dh, theta, start_pos + T, factors, magnitude, device=emb.device)
 
     x = plain_embedding(emb, tokens, s_in)
     for l in range(L):
@@ -200,7 +201,7 @@ def plain_forward(cfg, weights, tokens, rnd=None, logit_scale_rule="reference", 
         act = rnd(plain_swiglu(gate, up))
         x = x + s_res * rnd(plain_linear(act, weights[p + "mlp.down_proj.weight"]))   # jiuge.cpp:249
     if rows is not None:                       # only these positions' logits (the step function's choice, jiuge.cpp:270-277)
-        x = x[torch.as_tensor(rows, dtype=torch.long)]
+        x = x[torch.as_tensor(rows, dtype=torch.long, device=x.device)]
     h = rnd(plain_rmsnorm(x, weights["model.norm.weight"], eps) * s_out)              # jiuge.py:198-201
     return plain_linear(h, head)                                                       # jiuge.cpp:264
 

@@ -784,3 +784,127 @@ def test_the_device_peak_measurements_run():
     from infinicore_infer_amd.kernels import peaks
     assert 500 < peaks.mfma_bf16_tflops(iters=2000, blocks_per_unit=4) < 5100
     assert 1.0 < peaks.read_tbs(megabytes=512, blocks_per_unit=8) < 16.5
+
+
+# ---------------------------------------------------------------------------
+# long contexts: the key counts and split counts that the benchmark's steps run with
+# ---------------------------------------------------------------------------
+def _paged_fast(k, v, page_size, dtype, seed=0, extra_pages=5):
+    """As _paged, without a loop over the tokens: shuffled pages, unused rows NaN."""
+    t, nkvh, dh = k.shape
+    n_pages = (t + page_size - 1) // page_size
+    g = torch.Generator().manual_seed(seed)
+    perm = torch.randperm(n_pages + extra_pages, generator=g)[:n_pages]
+    pad = n_pages * page_size - t
+
+    def plane(x):
+        x = torch.cat([x.to(dtype), torch.full((pad, nkvh, dh), float("nan")).to(dtype)]) if pad else x.to(dtype)
+        out = torch.full((n_pages + extra_pages, nkvh, page_size, dh), float("nan")).to(dtype)
+        out[perm] = x.reshape(n_pages, page_size, nkvh, dh).permute(0, 2, 1, 3)
+        return out
+    return plane(k), plane(v), perm.to(torch.int32)
+
+
+@pytest.mark.parametrize("n_split", [8, 16, 32])
+@pytest.mark.parametrize("keys", [4100, 16500])
+@pytest.mark.parametrize("dtype,nh,nkvh,dh,page", [(torch.bfloat16, 6, 6, 64, 64), (torch.bfloat16, 6, 2, 64, 16),
+                                                   (torch.bfloat16, 16, 1, 128, 64), (torch.float32, 4, 4, 64, 64),
+                                                   (torch.float32, 4, 2, 128, 32)])
+def test_attention_decode_over_long_contexts(dtype, nh, nkvh, dh, page, keys, n_split):
+    """Single-token rows over 4,100 and 16,500 keys in 8, 16 and 32 splits (what the cost model chooses for the
+    benchmark's steps).  Random rows against the plain attention; and rows that must find ONE key: query i and key
+    p_i carry a large component along a direction of their own, so row i's output is value row p_i or the kernel has
+    missed that key.  The keys to find lie at the first and last position, at page edges and on both sides of every
+    boundary between two splits."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(keys + n_split)
+    scale = 1.0 / math.sqrt(dh)
+    per = (keys + n_split - 1) // n_split
+    needles = sorted({0, 1, page - 1, page, keys - 1, keys - 2, keys - page, keys // 2}
+                     | {min(keys - 1, s * per + o) for s in range(1, n_split, max(1, n_split // 8)) for o in (-1, 0)})[:dh // 2]
+    k = torch.randn(keys, nkvh, dh, generator=g) * 0.5
+    v = torch.randn(keys, nkvh, dh, generator=g)
+    n_rand = 5
+    q = torch.randn(n_rand + len(needles), nh, dh, generator=g) * 0.5
+    q[n_rand:] *= 0.05
+    for i, p in enumerate(needles):            # direction i: element 2 i of every head
+        k[p, :, 2 * i] = 30.0
+        q[n_rand + i, :, 2 * i] = 30.0         # score 900 / sqrt(dh) >= 79 against the others' few units
+    kc, vc, bt = _paged_fast(k, v, page, dtype, seed=keys)
+    R = q.shape[0]
+    # the random rows see contexts of different lengths; the others see all keys
+    ctx = [keys, keys - 1, keys - page, keys // 3, page + 1][:n_rand] + [keys] * len(needles)
+    btd = bt[None].repeat(R, 1).contiguous().to(DEV)
+    tr = torch.arange(R, dtype=torch.int32, device=DEV)
+    ps = torch.tensor([c - 1 for c in ctx], dtype=torch.int32, device=DEV)
+    qd = q.to(dtype).reshape(R, nh * dh).to(DEV)
+    out = torch.zeros_like(qd)
+    pa = torch.empty(R * nh * n_split * dh, device=DEV)
+    pm = torch.empty(R * nh * n_split * 2, device=DEV)
+    ops.attention_decode(qd, out, kc.to(DEV), vc.to(DEV), btd, None, R, tr, ps, pa, pm, nh, nkvh, dh, page, scale, 0, n_split)
+    got = out.float().cpu().reshape(R, nh, dh)
+    kd, vd = k.to(dtype).to(DEV), v.to(dtype).to(DEV)
+    for r in range(n_rand):
+        want = P.plain_attention(q[r:r + 1].to(dtype).to(DEV), kd[:ctx[r]], vd[:ctx[r]], scale, ctx[r] - 1)
+        _close(got[r], want[0].cpu(), dtype, factor=3)
+    for i, p in enumerate(needles):
+        want = v[p].to(dtype).float()          # [nkvh, dh]; head h reads kv head h // (nh / nkvh)
+        for h in range(nh):
+            err = float((got[n_rand + i, h] - want[h // (nh // nkvh)]).abs().max())
+            assert err < 0.05, "the key at position %d of %d (%d splits) was not found by head %d: off by %.3g" % (p, keys, n_split, h, err)
+
+
+@pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 64), (6, 2, 64, 16), (4, 4, 128, 64), (8, 1, 128, 32)])
+@pytest.mark.parametrize("past,new,parts", [(0, 4096, None), (0, 4096, (2, 32)), (3584, 512, (4, 16)), (3000, 1096, (3, 22))])
+def test_attention_prefill_walks_of_4096_keys(nh, nkvh, dh, page, past, new, parts):
+    """A prompt of 4,096 tokens whole (64 key tiles in the longest walk, whole and cut into parts), and portions after a
+    long past.  Against the plain attention; and, as above, query rows that must each find one key of their own: at
+    position 0, on both sides of tile and part boundaries, and the row's own position (the diagonal)."""
+    ops = _ops()
+    g = torch.Generator().manual_seed(past + new + nh)
+    t = past + new
+    scale = 1.0 / math.sqrt(dh)
+    k = torch.randn(t, nkvh, dh, generator=g) * 0.5
+    v = torch.randn(t, nkvh, dh, generator=g)
+    q = torch.randn(new, nh, dh, generator=g) * 0.5
+    part_keys = 64 * (parts[1] if parts else 16)
+    rows = sorted({0, 1, 127, 128, new - 1, new - 2, new // 2, new - 129})[:8]
+    needles = {}
+    for i, r in enumerate(rows):               # query row r (position past + r) must find key p
+        pos = past + r
+        cand = [0, pos, max(0, pos - 1), min(pos, part_keys - 1), min(pos, part_keys), pos // 2, max(0, pos - 64), min(pos, 63)]
+        needles[r] = cand[i % len(cand)]
+    used = {}
+    for i, (r, p) in enumerate(needles.items()):
+        if p in used:                          # two rows after the same key share its direction
+            d = used[p]
+        else:
+            d = used[p] = 2 * len(used)
+            k[p, :, d] = 30.0
+        q[r] *= 0.05
+        q[r, :, d] = 30.0
+    kc, vc, bt = _paged_fast(k, v, page, torch.bfloat16, seed=t)
+    qd = q.to(torch.bfloat16).reshape(new, nh * dh).to(DEV)
+    out = torch.zeros_like(qd)
+    tile_rows = ops.attention_prefill_tile_rows()
+    tiles = []
+    for o in range(0, new, tile_rows):
+        tiles += [0, o, min(tile_rows, new - o), past + o]
+    tl = torch.tensor(tiles, dtype=torch.int32, device=DEV).view(-1, 4)
+    btd = bt[None].contiguous().to(DEV)
+    if parts:
+        scratch = torch.full((ops.attention_prefill_scratch_floats(tl.shape[0], nh, dh, parts[0]),), float("nan"), device=DEV)
+        counters = torch.zeros(ops.attention_prefill_counter_ints(), dtype=torch.int32, device=DEV)
+        ops.attention_prefill(qd, out, kc.to(DEV), vc.to(DEV), btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, 0, 1,
+                              parts=parts[0], part_len=parts[1], scratch=scratch, counters=counters)
+        assert int(counters.abs().sum()) == 0
+    else:
+        ops.attention_prefill(qd, out, kc.to(DEV), vc.to(DEV), btd, tl, tl.shape[0], nh, nkvh, dh, page, scale, 0)
+    want = P.plain_attention(q.to(torch.bfloat16).to(DEV), k.to(torch.bfloat16).to(DEV), v.to(torch.bfloat16).to(DEV), scale, past)
+    _close(out.float().cpu().reshape(new, nh, dh), want.cpu(), torch.bfloat16, factor=3)
+    got = out.float().cpu().reshape(new, nh, dh)
+    for r, p in needles.items():
+        vp = v[p].to(torch.bfloat16).float()
+        for h in range(nh):
+            err = float((got[r, h] - vp[h // (nh // nkvh)]).abs().max())
+            assert err < 0.05, "query row %d (position %d) did not find the key at position %d: off by %.3g" % (r, past + r, p, err)
