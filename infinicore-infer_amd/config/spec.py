@@ -22,12 +22,15 @@ class PartSpec:
 
 @dataclass(frozen=True)
 class LayerSpec:
-    """A layer = a block arrangement over a mixer and a feed-forward."""
+    """A layer = a block arrangement over the parts it names.  Which parts a layer must have is the
+    block kind's question: the pre-norm residual block wants a mixer with its norm and takes a
+    feed-forward with its norm or none (a stack of mixers alone); another arrangement (one norm
+    shared by mixer and feed-forward, a feed-forward alone) names what it uses and leaves the rest None."""
     block: PartSpec
-    mixer: PartSpec
-    mixer_norm: PartSpec
-    feed_forward: PartSpec
-    feed_forward_norm: PartSpec
+    mixer: Optional[PartSpec] = None
+    mixer_norm: Optional[PartSpec] = None
+    feed_forward: Optional[PartSpec] = None
+    feed_forward_norm: Optional[PartSpec] = None
 
 
 @dataclass(frozen=True)

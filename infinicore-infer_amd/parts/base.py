@@ -244,7 +244,8 @@ class Block(Part):
     ``(y, alpha)``; a block may hand its last add on to the next block's norm."""
     category = "block"
 
-    def __init__(self, name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm):
+    def __init__(self, name, runtime, mixer=None, mixer_norm=None, feed_forward=None, feed_forward_norm=None):
+        """Any of the four may be None: a layer names the parts its arrangement uses (a subclass says which it needs)."""
         super().__init__(name, runtime)
         self.mixer = mixer
         self.mixer_norm = mixer_norm
@@ -252,7 +253,7 @@ class Block(Part):
         self.feed_forward_norm = feed_forward_norm
 
     def sub_parts(self):
-        return (self.mixer, self.mixer_norm, self.feed_forward, self.feed_forward_norm)
+        return tuple(p for p in (self.mixer, self.mixer_norm, self.feed_forward, self.feed_forward_norm) if p is not None)
 
     # A block with ``fuses_successor`` is called as forward(x, pending, ctx, cache, successor=norm):
     # ``successor`` is the norm that whoever runs next applies first (None: unknown or not splittable),

@@ -24,10 +24,11 @@ class DecoderModel:
         self.embedding = build_part("embedding", spec.embedding, runtime, memo)
         self.layers = []
         for ls in spec.layers:
-            mixer = build_part("mixer", ls.mixer, runtime, memo)
-            ffn = build_part("feed_forward", ls.feed_forward, runtime, memo)
-            n1 = build_part("norm", ls.mixer_norm, runtime, memo)
-            n2 = build_part("norm", ls.feed_forward_norm, runtime, memo)
+            opt = lambda category, spec: None if spec is None else build_part(category, spec, runtime, memo)
+            mixer = opt("mixer", ls.mixer)
+            ffn = opt("feed_forward", ls.feed_forward)
+            n1 = opt("norm", ls.mixer_norm)
+            n2 = opt("norm", ls.feed_forward_norm)
             from .base import _REGISTRY
             try:
                 block_cls = _REGISTRY["block"][ls.block.kind]
@@ -57,8 +58,8 @@ class DecoderModel:
         for e in self.schedule:
             if e.writes_cache:
                 continue
-            wn = self.layers[writers[e.cache]].mixer.cache_need()
-            rn = self.layers[e.layer].mixer.cache_need()
+            wn = self._cache_need_of(writers[e.cache])
+            rn = self._cache_need_of(e.layer)
             if not (wn.paged and rn.paged):
                 continue
             if (rn.planes, rn.n_kv_heads, rn.head_dim) != (wn.planes, wn.n_kv_heads, wn.head_dim):
@@ -105,12 +106,16 @@ class DecoderModel:
         self.load_weights(tensors)
 
     # ---- cache needs ------------------------------------------------------------------
+    def _cache_need_of(self, layer: int) -> CacheNeed:
+        mixer = self.layers[layer].mixer
+        return CacheNeed() if mixer is None else mixer.cache_need()       # a layer without a mixer keeps nothing
+
     def cache_needs(self) -> List[CacheNeed]:
         """One need per cache slot, in slot order."""
         n = self.spec.num_cache_slots()
         needs = [CacheNeed() for _ in range(n)]
         for slot, layer in self._writers.items():
-            needs[slot] = self.layers[layer].mixer.cache_need()
+            needs[slot] = self._cache_need_of(layer)
         return needs
 
     def weight_bytes(self) -> int:

@@ -704,3 +704,126 @@ def test_toy_architecture_with_a_one_plane_latent_cache_and_a_state_in_one_mixer
     out = eng.step([StepEntry("dst", toks[70:], list(range(len(toks) - 70)))])
     err = float((out.cpu().double() - ref["z2"][70:]).abs().max() / ref["z2"].abs().max())
     assert err < 1e-4, err
+
+
+# ---------------------------------------------------------------------------
+# a fourth toy architecture: layers that leave parts out.  A layer of a mixer alone (no feed-forward, no second
+# norm) under the package's pre-norm block; and a block arrangement defined here that shares ONE norm between its
+# mixer and its feed-forward (both read norm(x), both are added to the stream)
+# ---------------------------------------------------------------------------
+def _register_toy_sparse_layers():
+    from infinicore_infer_amd.config import LayerSpec, ModelSpec, PartSpec, default_schedule, register_architecture
+    from infinicore_infer_amd.kernels import ops
+    from infinicore_infer_amd.parts import Block, register_part
+
+    @register_part("block", "toy_parallel_one_norm")
+    class ParallelBlock(Block):
+        """x += a * (mixer(norm(x)) + ffn(norm(x))): one norm, no feed_forward_norm."""
+
+        def __init__(self, name, runtime, mixer=None, mixer_norm=None, feed_forward=None, feed_forward_norm=None, a=1.0):
+            super().__init__(name, runtime, mixer, mixer_norm, feed_forward, feed_forward_norm)
+            assert feed_forward_norm is None and None not in (mixer, mixer_norm, feed_forward)
+            self.a = float(a)
+
+        def forward(self, x, pending, ctx, cache):
+            if pending is not None:
+                ops.residual_add(x, pending[0], pending[1])
+            h = ctx.ws.buffer("toy_par_normed", tuple(x.shape), self.runtime.dtype)
+            self.mixer_norm.forward(x, h)
+            y = self.mixer.forward(h, ctx, cache)
+            ops.residual_add(x, y, self.a)
+            return (self.feed_forward.forward(h, ctx), self.a)          # the second add is left owed, as the package's block does
+
+    class SparseConfig:
+        def __init__(self, cfg):
+            self.cfg = cfg
+
+        @classmethod
+        def from_dict(cls, cfg, **kw):
+            return cls(cfg)
+
+        def model_spec(self):
+            c = self.cfg
+            d, nh, nkvh, dh = c["hidden"], c["heads"], c["kv_heads"], c["head_dim"]
+            rot = PartSpec("rotary", "", {"head_dim": dh, "theta": 500.0, "max_positions": c["max_pos"]})
+            norm = lambda p: PartSpec("rmsnorm", p, {"size": d, "eps": 1e-5})
+            ffn = lambda p: PartSpec("swiglu", p, {"hidden_size": d, "intermediate_size": c["inter"]})
+            attn = lambda p: PartSpec("attention", p, {"hidden_size": d, "num_heads": nh, "num_kv_heads": nkvh, "head_dim": dh,
+                                                       "softmax_scale": dh ** -0.5, "position_encoding": rot})
+            pre = lambda p: PartSpec("prenorm_residual", p, {"residual_scale": 0.7})
+            layers = [
+                LayerSpec(pre("l0."), attn("l0.att."), norm("l0.n1.")),                                   # a mixer alone
+                LayerSpec(pre("l1."), attn("l1.att."), norm("l1.n1.")),                                   # and another
+                LayerSpec(pre("l2."), attn("l2.att."), norm("l2.n1."), ffn("l2.ffn."), norm("l2.n2.")),   # the usual layer
+                LayerSpec(PartSpec("toy_parallel_one_norm", "l3.", {"a": 0.5}), attn("l3.att."), norm("l3.n."), ffn("l3.ffn.")),
+                LayerSpec(pre("l4."), attn("l4.att."), norm("l4.n1.")),                                   # a mixer alone before the head
+            ]
+            return ModelSpec("toy-sparse", c["vocab"], d, c["max_pos"],
+                             PartSpec("embedding", "emb.", {"vocab_size": c["vocab"], "hidden_size": d, "scale": 3.0}),
+                             layers, default_schedule(len(layers)), norm("final."),
+                             PartSpec("lm_head", "head.", {"vocab_size": c["vocab"], "hidden_size": d, "logit_scale": 1.0}))
+
+    register_architecture(["toy-sparse-arch"], SparseConfig)
+
+
+def _toy_sparse_plain(model, cfg, tokens, rnd=None):
+    rnd = rnd or (lambda t: t)
+    T, d, nh, nkvh, dh = len(tokens), cfg["hidden"], cfg["heads"], cfg["kv_heads"], cfg["head_dim"]
+    half = dh // 2
+    cpu = lambda t: t.detach().cpu().double()
+    sin, cos = P.plain_rope_tables(dh, 500.0, T)
+
+    def rope(x):
+        s, c = sin[:T, None, :], cos[:T, None, :]
+        return torch.cat([x[..., :half] * c - x[..., half:] * s, x[..., :half] * s + x[..., half:] * c], -1)
+
+    def attention(blk, h):
+        qkv = rnd(P.plain_linear(h, cpu(blk.mixer.w_qkv)))
+        q = rnd(rope(qkv[:, :nh * dh].reshape(T, nh, dh)))
+        k = rnd(rope(qkv[:, nh * dh:(nh + nkvh) * dh].reshape(T, nkvh, dh)))
+        v = qkv[:, (nh + nkvh) * dh:].reshape(T, nkvh, dh)
+        a = rnd(P.plain_attention(q, k, v, dh ** -0.5, 0, None)).reshape(T, nh * dh)
+        return rnd(P.plain_linear(a, cpu(blk.mixer.w_o)))
+
+    def ffn(blk, h):
+        gu = rnd(P.plain_linear(h, cpu(blk.feed_forward.w_gate_up)))
+        di = gu.shape[1] // 2
+        return rnd(P.plain_linear(rnd(P.plain_swiglu(gu[:, :di], gu[:, di:])), cpu(blk.feed_forward.w_down)))
+
+    x = P.plain_embedding(cpu(model.embedding.table), tokens, 3.0)
+    for blk in model.layers:
+        h = rnd(P.plain_rmsnorm(x, cpu(blk.mixer_norm.weight), 1e-5))
+        if type(blk).__name__ == "ParallelBlock":
+            x = x + 0.5 * attention(blk, h) + 0.5 * ffn(blk, h)
+            continue
+        x = x + 0.7 * attention(blk, h)
+        if blk.feed_forward is not None:
+            x = x + 0.7 * ffn(blk, rnd(P.plain_rmsnorm(x, cpu(blk.feed_forward_norm.weight), 1e-5)))
+    return P.plain_linear(rnd(P.plain_rmsnorm(x, cpu(model.final_norm.weight), 1e-5)), cpu(model.head.weight))
+
+
+@pytest.mark.parametrize("dtype,tol", [(torch.float32, 1e-4), (torch.bfloat16, H.BF16_TOL)])
+def test_toy_architecture_whose_layers_leave_parts_out(dtype, tol):
+    """Layers of a mixer alone under the package's own block (in bfloat16 with few rows their adds and norms still go
+    into the products on either side: the mixer's last projection hands half-normed rows to the next layer's mixer,
+    or to the head), and a block defined here with one norm for both its parts."""
+    from infinicore_infer_amd.config import config_from_dict
+    from infinicore_infer_amd.engine import Engine
+    from infinicore_infer_amd.parts import Runtime, build_model
+    from infinicore_infer_amd.weights import init_random_weights
+    _register_toy_sparse_layers()
+    cfg = {"model_type": "toy-sparse-arch", "vocab": 83, "hidden": 64, "heads": 4, "kv_heads": 2, "head_dim": 32,
+           "inter": 96, "max_pos": 192}
+    model = build_model(config_from_dict(cfg).model_spec(), Runtime(dtype, DEV))
+    init_random_weights(model, seed=17, std=0.12, norm_std=0.1, tie=False)
+    assert [l.feed_forward is None for l in model.layers] == [True, True, False, False, True]
+    assert model.layers[3].feed_forward_norm is None and len(model.cache_needs()) == 5
+    requests = {"s%d" % i: H.random_tokens(83, n, 80 + i) for i, n in enumerate([60, 21, 130, 7])}
+    rnd = P.round_bf16 if dtype == torch.bfloat16 else None
+    ref = {rid: _toy_sparse_plain(model, cfg, toks, rnd) for rid, toks in requests.items()}
+    for maker in (H.trace_whole, H.trace_last_one_by_one, H.trace_mixed):
+        steps, max_tokens = maker(requests)
+        eng = Engine(model, max_tokens=max_tokens, page_size=16, max_requests=4)
+        assert eng.native is None                      # a layer without a feed-forward has no native description
+        H.compare(H.run_trace(eng, steps), ref, tol, "toy sparse layers %s" % maker.__name__, steps=steps)
+        eng.cache.check_invariants()

@@ -340,7 +340,7 @@ def test_command_line_generates_what_the_plain_implementation_does(tmp_path, nam
     # two prompts together through the scheduler, random weights drawn from a configuration file
     conf = tmp_path / "conf.json"
     conf.write_text(json.dumps(dict(cfg, torch_dtype=dname)))
-    cmd = [sys.executable, "-m", "infinicore_infer_amd.minicpm", "--amd", "--random-weights", "--config", str(conf),
+    cmd = [sys.executable, "-m", "infinicore_infer_amd.causal_lm", "--amd", "--random-weights", "--config", str(conf),
            "--weights-seed", "6", "--weights-std", str(H.CONFIGS[name][1]["std"]),
            "--weights-norm-std", str(H.CONFIGS[name][1]["norm_std"]), "--max-new-tokens", "5",
            "--page-size", "32", "--num-pages", "8", "--chunk-size", "8", "--max-batch-tokens", "12"]

@@ -213,7 +213,7 @@ def test_a_task_whose_limit_lies_beyond_the_models_positions_ends_with_length():
 def test_command_line_arguments():
     """The command line's surface: the reference's positional form (scripts/jiuge.py:646-677) and the
     options beside it; parsing needs no GPU."""
-    from infinicore_infer_amd.minicpm import _parse
+    from infinicore_infer_amd.causal_lm import _parse
     path, ndev, a = _parse(["--amd", "/m", "1", "--prompt-ids", "1,2", "--prompt-ids", "3", "--max-new-tokens", "4",
                             "--top-k", "5", "--top-p", "0.5", "--chunk-size", "8", "--max-batch-tokens", "16",
                             "--num-pages", "9", "--page-size", "32", "--dtype", "float32"])
