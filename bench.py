@@ -33,6 +33,13 @@ MODEL = dict(
     scale_emb=12, dim_model_base=256, scale_depth=1.4, tie_word_embeddings=True, eos_token_id=2)
 # Two further shapes for --shape: MiniCPM-1B-shaped (deep, narrow, 3 query heads per kv head) and
 # MiniCPM4-8B/FM9G-8B-shaped (16 query heads per kv head, head size 128, longrope).  The default run is 2b.
+def _seeded_factors(seed, n=64):
+    """Long-context rotary factors drawn from the seed, uniform in [1, 4]."""
+    import random
+    rng = random.Random(seed)
+    return [1.0 + 3.0 * rng.random() for _ in range(n)]
+
+
 SHAPES = {
     "2b": MODEL,
     "1b": dict(MODEL, vocab_size=73440, hidden_size=1536, num_hidden_layers=52, num_attention_heads=24,
@@ -41,8 +48,7 @@ SHAPES = {
                num_key_value_heads=2, intermediate_size=16384, rms_norm_eps=1e-6, tie_word_embeddings=False,
                max_position_embeddings=32768,
                rope_scaling=dict(type="longrope", original_max_position_embeddings=32768,
-                                 short_factor=[1.0 + 3.0 * i / 63 for i in range(64)],
-                                 long_factor=[1.0 + 3.0 * i / 63 for i in range(64)])),
+                                 short_factor=_seeded_factors(1), long_factor=_seeded_factors(2))),
 }
 PROMPT = 2048
 BATCH = 8
@@ -53,6 +59,13 @@ def _sync():
     torch.cuda.synchronize()
 
 
+DTYPE = torch.bfloat16          # --dtype float32: the whole model in true 32-bit (weights, activations, cache, products)
+
+
+def _elem_bytes():
+    return 2 if DTYPE == torch.bfloat16 else 4
+
+
 def build_engine(layers, max_tokens, max_requests, page_size):
     from infinicore_infer_amd.config import config_from_dict
     from infinicore_infer_amd.engine import Engine
@@ -60,7 +73,7 @@ def build_engine(layers, max_tokens, max_requests, page_size):
     from infinicore_infer_amd.weights import init_random_weights
     cfg = dict(MODEL, num_hidden_layers=layers or MODEL["num_hidden_layers"])
     conf = config_from_dict(cfg)
-    model = build_model(conf.model_spec(), Runtime(dtype=torch.bfloat16, device="cuda:0"))
+    model = build_model(conf.model_spec(), Runtime(dtype=DTYPE, device="cuda:0"))
     init_random_weights(model, seed=0, std=WEIGHT_STD, tie=bool(cfg.get("tie_word_embeddings", True)))
     return Engine(model, max_tokens=max_tokens, page_size=page_size, max_requests=max_requests), conf
 
@@ -70,8 +83,9 @@ def model_numbers(conf):
     d, L, di, V = conf.hidden_size, conf.num_hidden_layers, conf.intermediate_size, conf.vocab_size
     nh, nkvh, dh = conf.num_attention_heads, conf.num_key_value_heads, conf.head_dim
     per_layer = (nh + 2 * nkvh) * dh * d + nh * dh * d + 3 * d * di
-    weight_bytes = 2 * (L * per_layer + V * d) + 4 * d * (2 * L + 1)      # the head's table once; embedding rows are negligible
-    kv_bytes_per_token = 2 * L * nkvh * dh * 2
+    eb = _elem_bytes()
+    weight_bytes = eb * (L * per_layer + V * d) + 4 * d * (2 * L + 1)      # the head's table once; embedding rows are negligible
+    kv_bytes_per_token = 2 * L * nkvh * dh * eb
 
     def prefill_flops(T):
         linear = 2.0 * T * L * per_layer
@@ -241,7 +255,7 @@ def run_mixed(args):
 
 
 def main():
-    global BATCH, MODEL, PROMPT
+    global BATCH, MODEL, PROMPT, DTYPE
     ap = argparse.ArgumentParser()
     ap.add_argument("--gpus", type=int, default=1)
     ap.add_argument("--steps", type=int, default=128)
@@ -261,7 +275,11 @@ def main():
     ap.add_argument("--no-tune", action="store_true", help="keep the library's default kernel choice for prefill products")
     ap.add_argument("--batch", type=int, default=BATCH, help="batch of the headline run (for profiling other points)")
     ap.add_argument("--eager", action="store_true", help="decode without HIP graphs (so that a profiler's counters attribute to kernels)")
+    ap.add_argument("--dtype", default="bfloat16", choices=["bfloat16", "float32"],
+                    help="float32: the whole model in true 32-bit (no reduced-precision matrix mode), against the fp32 peak")
     args = ap.parse_args()
+    DTYPE = {"bfloat16": torch.bfloat16, "float32": torch.float32}[args.dtype]
+    dname = "bf16" if DTYPE == torch.bfloat16 else "fp32"
     if args.gpus != 1:
         print("bench.py: this engine runs on one GPU; --gpus %d is not supported" % args.gpus)
         return 2
@@ -312,7 +330,7 @@ def main():
         "metric": "decode tokens/s, batch %d, %d-token prompts (MiniCPM-%s-shaped)" % (BATCH, PROMPT, args.shape.upper()),
         "value": round(value, 1), "unit": "tokens/s", "n_gpus": 1, "steps": args.steps, "warmup": args.warmup,
         "ms_per_step": round(ms, 4), "higher_is_better": True, "scaling": "weak", "vs_baseline": None,
-        "dtype": "bf16", "data": "synthetic (seeded random weights N(0,0.1) and token ids)",
+        "dtype": dname, "data": "synthetic (seeded random weights N(0,0.1) and token ids)",
         "config": {
             "model": "MiniCPM-%s-shaped" % args.shape.upper(), "layers": conf.num_hidden_layers, "layers_of_config": MODEL["num_hidden_layers"],
             "hidden": conf.hidden_size, "heads": conf.num_attention_heads, "kv_heads": conf.num_key_value_heads,
@@ -323,10 +341,16 @@ def main():
             "decode_launch": "eager" if args.eager else "hip graph", "decode_loop": "direct" if args.direct else "scheduler",
         },
         "prefill": {"value": round(PROMPT / t_pf, 1), "tokens": PROMPT, "ms": round(t_pf * 1e3, 3),
-                    "frac": round(pf_flops / t_pf / (PEAK_TFLOPS["bf16"] * 1e12), 4)},
+                    "frac": round(pf_flops / t_pf / (PEAK_TFLOPS[dname] * 1e12), 4)},
         "roofline": {"bound": "hbm", "achieved": round(achieved, 1), "peak": HBM_PEAK_GBS, "unit": "GB/s",
                      "frac": round(achieved / HBM_PEAK_GBS, 4)},
         "points": {("decode_b%d" % b): round(b / results[b][0], 1) for b in batches if b != BATCH},
+        # every point's step against the same bound: the bytes it has to read (weights once, the live requests' cache) / its time
+        "points_roofline": {("decode_b%d" % b): {
+            "ms": round(results[b][0] * 1e3, 4), "context": round(results[b][1], 1),
+            "achieved": round((weight_bytes + b * results[b][1] * kv_per_tok) / results[b][0] / 1e9, 1),
+            "frac": round((weight_bytes + b * results[b][1] * kv_per_tok) / results[b][0] / 1e9 / HBM_PEAK_GBS, 4)}
+            for b in batches},
     }
     print(json.dumps(out))
     return 0
