@@ -392,9 +392,14 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         }
 }
 
+// bfloat16: the kernel above.  float32: the true-float32 kernel of attn_prefill_f32.hip (same tiles, one wave group, walks never cut).
 IC_EXPORT int ic_attn_prefill_supported(int dtype, int dh, int page_size) {
-    return dtype == IC_BF16 && (dh == 64 || dh == 128) && page_size > 0 && (page_size & (page_size - 1)) == 0;
+    return (dtype == IC_BF16 || dtype == IC_F32) && (dh == 64 || dh == 128) && page_size > 0 && (page_size & (page_size - 1)) == 0;
 }
+
+int ic_attn_prefill_f32_launch(const void* q, int q_stride, void* out, int out_stride, const void* kcache, const void* vcache,
+                               const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh,
+                               int page_shift, float scale, int window, hipStream_t stream);
 
 IC_EXPORT int ic_attn_prefill_tile_rows() { return kPfRows; }
 IC_EXPORT int ic_attn_prefill_counter_ints() { return kPfCounters; }
@@ -447,6 +452,9 @@ IC_EXPORT int ic_attn_prefill_split(const void* q, int q_stride, void* out, int 
     int page_shift = 0;
     while ((1 << page_shift) < page_size) ++page_shift;
     if (nh <= 0 || nkvh <= 0 || nh % nkvh || page_size <= 0 || nh > 65535 || groups < 0 || groups > 2) return IC_ERR_ARG;
+    if (dtype == IC_F32)                                  // (groups, parts and scratch do not apply: its walks are never cut)
+        return ic_attn_prefill_f32_launch(q, q_stride, out, out_stride, kcache, vcache, block_tables, bt_stride, tiles, n_tiles, nh,
+                                          nkvh, dh, page_shift, scale, window, stream);
     if (q_stride % 8 || out_stride % 4 || ((uintptr_t)q & 15) || ((uintptr_t)out & 7) ||
         ((uintptr_t)kcache & 15) || ((uintptr_t)vcache & 15) || ((uintptr_t)tiles & 15)) return IC_ERR_ARG;
     if (parts < 1) parts = 1;

@@ -42,7 +42,8 @@ int ic_attn_generic(const void* q, int q_stride, void* out, int out_stride, int 
 // Split-key kernel for single new tokens.  part_acc: float32 [n_tok, nh, nsplit, dh]; part_ml: float32 [n_tok, nh, nsplit, 2]; nsplit <= 64.
 int ic_attn_decode_supported(int dtype, int dh);
 int ic_attn_decode(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tok_list, const int* token_req, const int* positions, float* part_acc, float* part_ml, int n_tok, int nh, int nkvh, int dh, int page_size, float scale, int window, int nsplit, hipStream_t stream);
-// Matrix-core kernel for prompt portions.  tiles: int32 [n_tiles, 4] = (request row, first token row, rows <= tile_rows, first position).
+// Matrix-core kernels for prompt portions (bfloat16; and true float32 with float32 matrix instructions, one wave group, walks never cut).
+// tiles: int32 [n_tiles, 4] = (request row, first token row, rows <= tile_rows, first position).
 int ic_attn_prefill_supported(int dtype, int dh, int page_size);
 int ic_attn_prefill_tile_rows();
 int ic_attn_prefill(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, hipStream_t stream);

@@ -7,8 +7,9 @@ P V, output projection.  Query head h uses key/value head h // (nh/nkvh)
 (jiuge.cpp:210-213).  Here the scores never reach memory: one of three kernels
 walks the cache with a float32 running softmax,
   * a split-key kernel for rows that are a request's single new token,
-  * a matrix-core kernel for prompt portions (bfloat16, head size 64 or 128),
-  * the general kernel for everything else and for float32 portions.
+  * a matrix-core kernel for prompt portions (head size 64 or 128; bfloat16, or true float32 with
+    float32 matrix instructions),
+  * the general kernel for everything else.
 """
 import torch
 

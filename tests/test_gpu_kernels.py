@@ -251,6 +251,16 @@ def test_attention_prefill_mfma(nh, nkvh, dh, page, window, groups):
 
 
 @pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (3, 1, 64, 32), (4, 2, 128, 16), (4, 4, 128, 64)])
+@pytest.mark.parametrize("window", [None, 100])
+def test_attention_prefill_in_true_float32(nh, nkvh, dh, page, window):
+    """Prompt portions in float32 on the matrix cores (float32 operands and accumulation): whole prompts, portions after a
+    past, tiles that end inside a page, two tokens, a window; to float32 accuracy against the plain attention."""
+    lens = [(0, 2), (0, 129), (130, 64), (64, 33), (15, 2), (257, 300), (5, 128), (700, 140)]
+    got, want = _attention_case(torch.float32, nh, nkvh, dh, page, lens, window, 33, "prefill")
+    _close(got, want, torch.float32, factor=3)
+
+
+@pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (3, 1, 64, 32), (4, 2, 128, 16), (4, 4, 128, 64)])
 @pytest.mark.parametrize("window", [None, 300])
 @pytest.mark.parametrize("parts", [(2, 1), (3, 2), (4, 1), (8, 3)])
 def test_attention_prefill_with_the_walk_over_the_keys_cut_into_parts(nh, nkvh, dh, page, window, parts):
@@ -334,7 +344,7 @@ def test_attention_special_cases():
 
 @pytest.mark.parametrize("impl,dtype", [("generic", torch.float32), ("generic", torch.bfloat16),
                                         ("decode", torch.float32), ("decode", torch.bfloat16),
-                                        ("prefill", torch.bfloat16)])
+                                        ("prefill", torch.bfloat16), ("prefill", torch.float32)])
 def test_attention_far_key_and_window_edge(impl, dtype):
     """One far key among hundreds is made to stand out (its score dwarfs the rest):
     the output must be its value row.  With a window, the key at its edge counts
