@@ -30,6 +30,7 @@ class CacheStorage:
                 self._slot_index[s] = (g, i)
         self.state: Dict[int, torch.Tensor] = {}               # cache slot -> [max_requests, ...]
         self._kv_views: Dict[int, tuple] = {}
+        self._copy_idx = None                                  # (pinned, device) page ids of copy_pages, kept between calls
 
     def add_state(self, slot: int, max_requests: int, shape, dtype) -> torch.Tensor:
         t = torch.zeros((max_requests,) + tuple(shape), dtype=dtype, device=self.device)
@@ -61,8 +62,18 @@ class CacheStorage:
             return
         from ..kernels import ops
         planes = self.group_planes[group]
-        idx = torch.tensor([list(src_pages), list(dst_pages)], dtype=torch.int32).to(self.device)
-        ops.copy_pages(planes, idx[0].contiguous(), idx[1].contiguous())
+        n = len(src_pages)
+        # page ids through a pinned buffer into device memory that is kept (grown to the largest copy asked for)
+        if self._copy_idx is None or self._copy_idx[0].shape[1] < n:
+            cap = max(n, 64)
+            self._copy_idx = (torch.empty(2, cap, dtype=torch.int32, pin_memory=True),
+                              torch.empty(2, cap, dtype=torch.int32, device=self.device))
+        host, dev = self._copy_idx
+        torch.cuda.current_stream().synchronize()          # the copy before has read the pinned buffer
+        host[0, :n] = torch.as_tensor(list(src_pages), dtype=torch.int32)
+        host[1, :n] = torch.as_tensor(list(dst_pages), dtype=torch.int32)
+        dev.copy_(host, non_blocking=True)
+        ops.copy_pages(planes, dev[0, :n], dev[1, :n])
 
     def copy_state(self, src_slot: int, dst_slot: int) -> None:
         for t in self.state.values():

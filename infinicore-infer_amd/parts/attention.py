@@ -99,7 +99,7 @@ class Attention(Mixer):
         width = (self.nh + 2 * (0 if self.shared_kv else self.nkvh)) * self.dh
         qkv = ctx.ws.buffer("qkv", (T, width), rt.dtype)
         if not self.pos_enc.project_rotate_store(h, self.w_qkv, qkv, ctx, cache, self.nh, nkv, self.dh):
-            linear(h, self.w_qkv, qkv, rt.gemm_impl)
+            linear(h, self.w_qkv, qkv, rt.gemm_impl, ws=ctx.ws)
             self.pos_enc.rotate_and_store(qkv, ctx, cache, self.nh, nkv, self.dh)
         out = ctx.ws.buffer("attn_out", (T, self.nh * self.dh), rt.dtype)
         self._attend(qkv, out, ctx, cache)
@@ -107,7 +107,7 @@ class Attention(Mixer):
         if fused is not None:
             return fused
         y = ctx.ws.buffer("mixer_out", (T, self.hidden_size), rt.dtype)
-        linear(out, self.w_o, y, rt.gemm_impl)
+        linear(out, self.w_o, y, rt.gemm_impl, ws=ctx.ws)
         return y
 
     def _key_splits(self, ctx) -> int:

@@ -109,10 +109,10 @@ class LMHead(Part):
         if isinstance(x, DeferredRows):
             # every row in order, the final norm half done: its row factors go into the product
             logits = ctx.ws.buffer("logits", (x.shape[0], self.vocab_size), torch.float32)
-            return linear(x, self.weight, logits, self.runtime.gemm_impl)     # the scale is in x (deferred_norm)
+            return linear(x, self.weight, logits, self.runtime.gemm_impl, ws=ctx.ws)     # the scale is in x (deferred_norm)
         n = rows.numel()
         h = ctx.ws.buffer("head_in", (n, self.hidden_size), self.runtime.dtype)
         final_norm.forward(x, h, rows=rows, out_scale=self.logit_scale)
         logits = ctx.ws.buffer("logits", (n, self.vocab_size), torch.float32)
-        linear(h, self.weight, logits, self.runtime.gemm_impl)
+        linear(h, self.weight, logits, self.runtime.gemm_impl, ws=ctx.ws)
         return logits

@@ -50,9 +50,11 @@ def own_kernel_applies(M, x_dtype, w_dtype, out_dtype, impl: str) -> bool:
     return impl == "auto" and ops.rule_own_product(x_dtype, w_dtype, out_dtype, M)
 
 
-def linear(x, w, out, impl: str = "auto", alpha: float = 1.0):
+def linear(x, w, out, impl: str = "auto", alpha: float = 1.0, ws=None):
     """out[M, N] = alpha * x[M, K] @ w[N, K]^T.  out may be float32 when x is bfloat16.  x may be
-    ``DeferredRows``: the row factors are applied to the result by the own kernel, or to x first."""
+    ``DeferredRows``: the row factors are applied to the result by the own kernel, or to x first.
+    ``ws``: the step's workspace, for the float32 copies that a matrix stored in 32-bit under a bfloat16
+    model needs (without it they are allocated by the call)."""
     if isinstance(x, DeferredRows):
         if own_kernel_applies(x.shape[0], x.dtype, w.dtype, out.dtype, impl):
             return ops.gemm_nt(x.values, w, out, alpha=alpha, row_factor=x.row_factor())
@@ -60,10 +62,16 @@ def linear(x, w, out, impl: str = "auto", alpha: float = 1.0):
     if w.dtype != x.dtype:
         # a matrix stored in 32-bit stays so: compute this product in float32
         # (w is the 32-bit one, so only the few activations are converted; no copy of the matrix is made)
+        def scratch(name, shape):
+            if ws is None:
+                return torch.empty(shape, dtype=torch.float32, device=out.device)
+            return ws.buffer(name, shape, torch.float32)
+        x32 = x if x.dtype == torch.float32 else scratch("linear_x32", tuple(x.shape)).copy_(x)
+        w32 = w if w.dtype == torch.float32 else w.to(torch.float32)
         if out.dtype == torch.float32:
-            return _library(x.to(torch.float32), w.to(torch.float32), out, alpha)
-        tmp = torch.empty(out.shape, dtype=torch.float32, device=out.device)
-        _library(x.to(torch.float32), w.to(torch.float32), tmp, alpha)
+            return _library(x32, w32, out, alpha)
+        tmp = scratch("linear_out32", tuple(out.shape))
+        _library(x32, w32, tmp, alpha)
         out.copy_(tmp)
         return out
     if own_kernel_applies(x.shape[0], x.dtype, w.dtype, out.dtype, impl):

@@ -72,11 +72,11 @@ class SwiGLU(FeedForward):
                 ops.gemm_nt(h, self.w_gate_up, act, swiglu_output=True)
         else:
             gate_up = ctx.ws.buffer("gate_up", (T, 2 * self.intermediate_size), rt.dtype)
-            linear(h, self.w_gate_up, gate_up, rt.gemm_impl)
+            linear(h, self.w_gate_up, gate_up, rt.gemm_impl, ws=ctx.ws)
             ops.swiglu(gate_up, act)
         fused = linear_tail(act, self.w_down, tail, ctx.ws, "ffn_tail", rt.gemm_impl)
         if fused is not None:
             return fused
         y = ctx.ws.buffer("ffn_out", (T, self.hidden_size), rt.dtype)
-        linear(act, self.w_down, y, rt.gemm_impl)
+        linear(act, self.w_down, y, rt.gemm_impl, ws=ctx.ws)
         return y
