@@ -105,6 +105,47 @@ def test_first_tokens(tmp_path_factory, name, dname, dtype, tol):
     H.compare(H.run_trace(engine, whole), ref, tol, "first tokens as one portion")
 
 
+@pytest.mark.parametrize("mode", ["last32", "chunks", "mixed"])
+@pytest.mark.parametrize("dname,dtype,tol", DTYPES)
+@pytest.mark.parametrize("name,gain", [("A", 9.0), ("C", 2.0), ("D", 2.0)])       # scores about two units apart
+def test_replay_modes_with_attention_that_picks_its_keys(tmp_path_factory, name, gain, dname, dtype, tol, mode):
+    """With weights of a few hundredths every score is near zero and attention is close to a plain mean of the values: a key
+    that is skipped, read from a neighbour's page or seen one position off would move the logits less than the tolerance.
+    Here the q and k projections are scaled up until the scores are about two units apart (much more and attention
+    turns into an argmax, which two correct bfloat16 computations resolve differently), so that every query picks a few
+    keys and what it picks depends on the rotation and on the exact position (and the values are scaled up so that what
+    attention adds weighs in the logits); then the replay modes again (single tokens
+    after a prompt, portions down to two tokens, mixed batches on pages that are used again)."""
+    import os
+    from safetensors.torch import save_file
+    from infinicore_infer_amd.engine import Engine
+    base = H.make_model_dir(tmp_path_factory.getbasetemp(), name)
+    folder = os.path.join(str(tmp_path_factory.getbasetemp()), "model_%s_peaked" % name)
+    if not os.path.isdir(folder):
+        os.makedirs(folder)
+        # (and the value projection by 4: in these tiny models the embedding dominates the residual stream, and what
+        # attention adds would otherwise move the logits by a few per cent at most)
+        sd = {k: ((v.float() * (gain if ("q_proj" in k or "k_proj" in k) else 4.0 if "v_proj" in k else 1.0)).to(v.dtype)).contiguous()
+              for k, v in H.load_state_dict(base).items()}
+        save_file(sd, os.path.join(folder, "model.safetensors"), metadata={"format": "pt"})
+        with open(os.path.join(base, "config.json")) as f, open(os.path.join(folder, "config.json"), "w") as g:
+            g.write(f.read())
+    cfg = H.CONFIGS[name][0]
+    sd = H.load_state_dict(folder)
+    requests = _requests(name, seed=3)
+    steps, max_tokens = MODES[mode](requests)
+    engine = Engine.from_dir(folder, dtype=dtype, max_tokens=max_tokens, page_size=16, max_requests=8)
+    ref = H.plain_logits(cfg, sd, requests, dtype == torch.bfloat16)
+    # the attention really is peaked: the plain model with the values of every other key swapped gives other logits
+    # (checked once, on the longest request, in float32)
+    if mode == "last32" and dtype == torch.float32:
+        flat = H.plain_logits(cfg, H.load_state_dict(base), {"r3": requests["r3"]}, False)["r3"]
+        assert float((flat - ref["r3"]).abs().max()) / float(ref["r3"].abs().max()) > 0.05
+    worst = H.compare(H.run_trace(engine, steps), ref, tol, "%s %s %s, peaked attention" % (name, dname, mode), steps=steps)
+    print("worst", worst)
+    engine.cache.check_invariants()
+
+
 @pytest.mark.parametrize("dname,dtype,tol", DTYPES)
 @pytest.mark.parametrize("name", ["A", "C"])
 def test_decoding_twenty_requests_at_once(tmp_path_factory, name, dname, dtype, tol):
