@@ -528,6 +528,9 @@ attn_decode_gqa_kernel(const uint16_t* __restrict__ q, int q_stride,
     }
 }
 
+// Grouped queries in bfloat16 run the matrix-core kernel: the one place that says so (the key-split rule asks here too).
+IC_EXPORT int ic_attn_decode_on_matrix_cores(int dtype, int n_heads, int n_kv_heads) { return dtype == IC_BF16 && n_heads != n_kv_heads; }
+
 template <typename T, int DH>
 static int launch_decode(const void* q, int q_stride, void* out, int out_stride, const void* kcache,
                          const void* vcache, const int* block_tables, int bt_stride, const int* tok_list,
@@ -541,7 +544,7 @@ static int launch_decode(const void* q, int q_stride, void* out, int out_stride,
     hipLaunchKernelGGL(KERNEL, grid, block, 0, stream, (const TQ*)q, q_stride, (const TQ*)kcache,           \
                        (const TQ*)vcache, block_tables, bt_stride, tok_list, token_req, positions, part_acc, \
                        part_ml, nh, nkvh, page_size, scale, window, nsplit, (TQ*)direct, out_stride)
-    if (nh != nkvh && sizeof(T) == 2) {
+    if (ic_attn_decode_on_matrix_cores(sizeof(T) == 2 ? IC_BF16 : IC_F32, nh, nkvh)) {
         if (staged) IC_DEC_LAUNCH((attn_decode_gqa_kernel<DH, true>), uint16_t);
         else IC_DEC_LAUNCH((attn_decode_gqa_kernel<DH, false>), uint16_t);
     } else if (nh == nkvh) {

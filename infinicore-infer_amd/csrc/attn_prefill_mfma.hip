@@ -438,6 +438,18 @@ IC_EXPORT int ic_attn_prefill_parts(int n_tiles, int nh, int dh, int max_keys, i
     return parts;
 }
 
+// The same question for a step: its largest position and the mixer's window (0: none) give the most keys a tile sees.
+// (float32 walks are never cut.)
+IC_EXPORT int ic_attn_prefill_parts_of_step(int dtype, int n_tiles, int nh, int dh, int max_position, int window, int compute_units, int* part_len) {
+    int keys = max_position + 1;
+    if (dtype != IC_BF16) {
+        if (part_len) *part_len = (keys + kPfKeys - 1) / kPfKeys;
+        return 1;
+    }
+    if (window > 0 && window + kPfRows < keys) keys = window + kPfRows;
+    return ic_attn_prefill_parts(n_tiles, nh, dh, keys, compute_units, part_len);
+}
+
 // tiles: int32 [n_tiles, 4] = (request row of block_tables, first token row, rows <= 128, position of the first row).
 // groups: 1 or 2 wave groups per query tile, 0 = chosen from the number of blocks.  parts > 1 (one group only): the grid
 // holds `parts` blocks per (tile, head) and a tile's walk is cut into up to that many parts of at least part_len key

@@ -111,7 +111,7 @@ struct IcDecoder {
 
     int splits_for(const IcStepBatch& b, const IcAttention& a) const {
         if (b.fixed_decode_splits > 0) return b.fixed_decode_splits;
-        const int matrix_cores = (meta.dtype == IC_BF16 && a.n_heads != a.n_kv_heads) ? 1 : 0;
+        const int matrix_cores = ic_attn_decode_on_matrix_cores(meta.dtype, a.n_heads, a.n_kv_heads);
         const int key[7] = {b.n_decode_rows, a.n_heads, a.n_kv_heads, a.head_dim, a.window, b.max_context, matrix_cores};
         if (memcmp(key, split_key, sizeof key) != 0) {
             split_answer = ic_attn_decode_splits(b.n_decode_rows, a.n_heads, a.n_kv_heads, a.head_dim, dtype_size(meta.dtype), a.window,
@@ -124,9 +124,7 @@ struct IcDecoder {
     // into how many parts the walks of a step's prompt tiles are cut (1: not at all), and key tiles per part
     int tile_parts_for(const IcStepBatch& b, const IcAttention& a, int* part_len) const {
         if (!meta.attention_counters) { if (part_len) *part_len = 0; return 1; }     // no counters: no cut
-        int keys = b.max_position + 1;
-        if (a.window > 0 && a.window + ic_attn_prefill_tile_rows() < keys) keys = a.window + ic_attn_prefill_tile_rows();
-        return ic_attn_prefill_parts(b.n_prefill_tiles, a.n_heads, a.head_dim, keys, meta.compute_units, part_len);
+        return ic_attn_prefill_parts_of_step(meta.dtype, b.n_prefill_tiles, a.n_heads, a.head_dim, b.max_position, a.window, meta.compute_units, part_len);
     }
 
     Workspace layout(const IcStepBatch& b) const {

@@ -41,6 +41,9 @@ int ic_rope_kv_write(void* qkv, int dtype, const int* positions, const float* co
 int ic_attn_generic(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* token_req, const int* positions, int T, int nh, int nkvh, int dh, int page_size, float scale, int window, hipStream_t stream);
 // Split-key kernel for single new tokens.  part_acc: float32 [n_tok, nh, nsplit, dh]; part_ml: float32 [n_tok, nh, nsplit, 2]; nsplit <= 64.
 int ic_attn_decode_supported(int dtype, int dh);
+// 1 when ic_attn_decode runs its grouped-query kernel on the matrix cores (bfloat16, several query heads per kv head): that
+// kernel wants other key splits than the one-head-per-wave kernel (the matrix_cores argument of ic_attn_decode_splits).
+int ic_attn_decode_on_matrix_cores(int dtype, int n_heads, int n_kv_heads);
 int ic_attn_decode(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tok_list, const int* token_req, const int* positions, float* part_acc, float* part_ml, int n_tok, int nh, int nkvh, int dh, int page_size, float scale, int window, int nsplit, hipStream_t stream);
 // Matrix-core kernels for prompt portions (bfloat16; and true float32 with float32 matrix instructions, one wave group, walks never cut).
 // tiles: int32 [n_tiles, 4] = (request row, first token row, rows <= tile_rows, first position).
@@ -59,6 +62,7 @@ int ic_attn_prefill_groups(const void* q, int q_stride, void* out, int out_strid
 long long ic_attn_prefill_scratch_floats(int n_tiles, int nh, int dh, int parts);
 int ic_attn_prefill_counter_ints();
 int ic_attn_prefill_parts(int n_tiles, int nh, int dh, int max_keys, int compute_units, int* part_len);
+int ic_attn_prefill_parts_of_step(int dtype, int n_tiles, int nh, int dh, int max_position, int window, int compute_units, int* part_len);   // max_keys from the step's largest position and the window
 int ic_attn_prefill_split(const void* q, int q_stride, void* out, int out_stride, int dtype, const void* kcache, const void* vcache, const int* block_tables, int bt_stride, const int* tiles, int n_tiles, int nh, int nkvh, int dh, int page_size, float scale, int window, int groups, int parts, int part_len, float* scratch, long long scratch_floats, int* counters, hipStream_t stream);
 
 // ---- gemm.hip ---------------------------------------------------------------------------------------

@@ -105,6 +105,7 @@ _SIGNATURES = {
     "ic_attn_prefill_groups": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _P],
     "ic_attn_prefill_scratch_floats": [_I, _I, _I, _I],
     "ic_attn_prefill_parts": [_I, _I, _I, _I, _I, _c.POINTER(_I)],
+    "ic_attn_prefill_parts_of_step": [_I, _I, _I, _I, _I, _I, _I, _c.POINTER(_I)],
     "ic_attn_prefill_split": [_P, _I, _P, _I, _I, _P, _P, _P, _I, _P, _I, _I, _I, _I, _I, _F, _I, _I, _I, _I, _P, _LL, _P, _P],
     "ic_attn_prefill_counter_ints": [],
     "ic_sample": [_P, _LL, _I, _I, _P, _P, _P, _P, _P, _P],
@@ -139,6 +140,7 @@ _SIGNATURES = {
     "ic_rule_tail": [_I, _I, _I, _I, _I, _I],
     "ic_rule_attention": [_I, _I, _I, _I, _I],
     "ic_rule_context_bucket": [_I],
+    "ic_attn_decode_on_matrix_cores": [_I, _I, _I],
     "ic_decoder_create": [_c.POINTER(IcDecoderMeta), _c.POINTER(IcLayer), _c.POINTER(IcRunEntry)],
     "ic_decoder_create_error": [],
     "ic_decoder_destroy": [_P],

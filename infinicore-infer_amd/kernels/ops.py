@@ -203,8 +203,8 @@ def attention_decode_supported(dtype, head_dim: int) -> bool:
 
 def attention_decode_on_matrix_cores(dtype, n_heads: int, n_kv_heads: int) -> bool:
     """True when attention_decode runs its grouped-query kernel (bfloat16, several query heads per
-    kv head): that kernel wants fewer key splits than the one-head-per-wave kernel."""
-    return dtype == torch.bfloat16 and n_heads != n_kv_heads
+    kv head): that kernel wants fewer key splits than the one-head-per-wave kernel (the library's rule)."""
+    return bool(get_lib().ic_attn_decode_on_matrix_cores(dtype_code(dtype), int(n_heads), int(n_kv_heads)))
 
 
 def attention_decode_splits(n_rows: int, n_heads: int, n_kv_heads: int, head_dim: int, elem_bytes: int, window: int,
@@ -254,6 +254,16 @@ def attention_prefill_parts(n_tiles: int, n_heads: int, head_dim: int, max_keys:
     part_len = ctypes.c_int(0)
     parts = get_lib().ic_attn_prefill_parts(int(n_tiles), int(n_heads), int(head_dim), int(max_keys), int(compute_units),
                                             ctypes.byref(part_len))
+    return int(parts), int(part_len.value)
+
+
+def attention_prefill_parts_of_step(dtype, n_tiles: int, n_heads: int, head_dim: int, max_position: int, window: int, compute_units: int):
+    """(parts, part_len) for a step whose largest position is ``max_position`` under a mixer's ``window`` (0: none);
+    float32 walks are never cut."""
+    import ctypes
+    part_len = ctypes.c_int(0)
+    parts = get_lib().ic_attn_prefill_parts_of_step(dtype_code(dtype), int(n_tiles), int(n_heads), int(head_dim), int(max_position), int(window or 0),
+                                                    int(compute_units), ctypes.byref(part_len))
     return int(parts), int(part_len.value)
 
 

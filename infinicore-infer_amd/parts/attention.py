@@ -147,10 +147,7 @@ class Attention(Mixer):
                                  self.window, n_split)
         if use_pre:
             # few blocks and long walks over the keys: the tiles' walks are cut into parts (the library's rule)
-            keys = ctx.max_position + 1
-            if self.window:
-                keys = min(keys, self.window + ops.attention_prefill_tile_rows())
-            parts, part_len = ops.attention_prefill_parts(n_tiles, self.nh, self.dh, keys, ctx.cu_count)
+            parts, part_len = ops.attention_prefill_parts_of_step(rt.dtype, n_tiles, self.nh, self.dh, ctx.max_position, self.window, ctx.cu_count)
             scratch = counters = None
             if parts > 1:
                 scratch = ctx.ws.buffer("attn_tile_parts", (ops.attention_prefill_scratch_floats(n_tiles, self.nh, self.dh, parts),),
