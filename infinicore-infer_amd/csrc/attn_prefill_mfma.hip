@@ -6,8 +6,9 @@
 // the two groups take the even and the odd key tiles of 64 and are merged through LDS at the
 // end: the longest query tile of a prompt, which sets the kernel's time when there are few
 // blocks, then walks half as many key tiles.  With many blocks GROUPS == 1 keeps more of them
-// resident and is faster.  Keys and values come through LDS as rows, 64 * GROUPS keys a step; the
-// next step is already on its way from memory while the current one is used.  The V^T operand is
+// resident and is faster.  Keys and values come through LDS as rows, 64 * GROUPS keys a step, loaded
+// from memory straight into LDS (no registers in between, one barrier a step); the next step's are on
+// their way into a second stage while the current one is used.  The V^T operand is
 // read with ds_read_b64_tr_b16, which transposes 16-bit elements across the lanes of a 16-lane
 // group on the way out of LDS (lane 16G + i receives, for e = 0..3, element i % 4 of the 8-byte
 // chunk that lane 16G + i / 4 + 4e pointed at).  Scores
@@ -32,6 +33,7 @@
 //
 // Cache layout of one layer: K and V planes [num_pages, n_kv_heads, page_size, head_dim].
 #include "common.h"
+#include <type_traits>
 
 // Arrival counters of the split walk, one per (tile, head), in memory of the caller's: zero before the first launch,
 // and put back to zero by the block that merges, so launches that follow each other on a stream share one buffer.
@@ -45,7 +47,6 @@ typedef short tr_v4s __attribute__((ext_vector_type(4)));
 constexpr int kPfWaveThreads = 256;   // four waves own the 128 rows of a query tile
 constexpr int kPfRows = 128;      // query rows per block
 constexpr int kPfKeys = 64;       // keys per tile
-constexpr int kPfPad = 8;         // elements of padding per LDS row
 constexpr int kPfMaxPages = 2048; // pages of one request whose ids are staged in LDS (else read from memory)
 
 union Frag8 {
@@ -63,18 +64,24 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
                          int parts, int part_len, float* __restrict__ scratch, int* __restrict__ counters) {
     constexpr int NC = DH / 16;           // 16-wide chunks of the head dimension
     constexpr int ND = DH / 32;           // 32-row tiles of O^T
-    constexpr int KS = DH + kPfPad;       // row stride of Ks (elements): 16-byte reads of 8 consecutive rows cover all banks
-    constexpr int VS = DH + 2 * kPfPad;   // row stride of Vs: the transposing 8-byte reads touch 4 rows at once, which must
-                                          // fall into different banks (a stride of 32 bytes mod 128; with KS two rows share one)
+    constexpr int CPR = DH / 8;           // 16-byte chunks of a row
     constexpr int kPfThreads = kPfWaveThreads * GROUPS;
     constexpr int STEP = kPfKeys * GROUPS;                 // keys staged per step
-    constexpr int NL = STEP * (DH / 8) / kPfThreads;       // 16-byte loads per thread per plane and step
-    constexpr int KT = kPfKeys * KS, VT = kPfKeys * VS;    // elements of one group's K and V tile
+    constexpr int NL = STEP * CPR / kPfThreads;            // 16-byte loads per thread per plane and step
+    constexpr int TILE = kPfKeys * DH;                     // elements of one group's K (or V) tile: rows without padding
+    constexpr int STAGE = 2 * GROUPS * TILE;               // a step's tiles: K of every group, then V of every group
     constexpr int MERGE_F = 2 + ND * 16;                   // floats a lane hands over at the end
-    static_assert(GROUPS == 1 || sizeof(uint16_t) * GROUPS * (KT + VT) >= sizeof(float) * 256 * MERGE_F, "merge buffer fits in the tiles");
-    __shared__ __attribute__((aligned(16))) uint16_t tilebuf[GROUPS * (KT + VT)];
-    uint16_t* const Ks_all = tilebuf;                      // [group][key][KS]
-    uint16_t* const Vs_all = tilebuf + GROUPS * KT;     // [group][key][VS]
+    static_assert(GROUPS == 1 || sizeof(uint16_t) * STAGE >= sizeof(float) * 256 * (2 + (ND / 2) * 16), "each half of the merge buffer fits in a stage");
+    // Two stages: the loads of the next step write one while the other is read.  They go from memory straight into LDS
+    // (global_load_lds_dwordx4: lane i of a wave writes 16 bytes at the wave's base + 16 i, no registers, no store
+    // instructions), so rows cannot be padded; instead the 16-byte chunks of row r sit at position (chunk ^ swz(r)), which a
+    // lane arranges by fetching the chunk that belongs where it writes.  With swz(r) = 2 (r % 4) + (r / 4) % 2 the 16-byte
+    // reads of 8 consecutive rows (K operand) and the transposing 8-byte reads of 4 consecutive rows x 32 bytes (V operand)
+    // each cover all banks once.
+    // (Two arrays, and the stage a compile-time constant wherever they are used: the compiler then knows that a load
+    // in flight into one does not touch what is read from the other, and does not wait for it before every LDS read.)
+    __shared__ __attribute__((aligned(16))) uint16_t stage0[STAGE];
+    __shared__ __attribute__((aligned(16))) uint16_t stage1[STAGE];
 
     __shared__ int pages[kPfMaxPages];
 
@@ -151,84 +158,84 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     const uint16_t* vbase = vcache + (size_t)kvh * head_stride;
     const size_t page_stride = (size_t)nkvh * head_stride;
 
-    // thread -> (key, octet), octets along lanes: a wave loads and stores whole rows of K and of V
-    uint4 kreg[NL], vreg[NL];
-    // PAGE64 (pages of 64 tokens and more): a 64-key tile lies in one page, so a step needs one page
-    // lookup per tile and every load is that tile's first row plus an offset the thread keeps.
-    constexpr int KPI = kPfThreads / (DH / 8);                // keys one pass of K loads covers (<= 64)
+    // What a thread loads in a step never changes: LDS chunk tid + i * threads of the step's K (and V) tiles, that is key
+    // `tkey` of the step's keys at chunk position idx % CPR, which holds the row's chunk `pos ^ swz(key)`.
+    auto swz = [](int row) -> int { return ((row & 3) << 1) | ((row >> 2) & 1); };
+    constexpr int KPI = kPfThreads / CPR;                     // keys one pass of loads covers (<= 64)
     static_assert(KPI <= kPfKeys && kPfKeys % KPI == 0, "a pass of loads stays inside a tile");
-    // what a thread loads in a step never changes: key `tkey` of the step's keys, at element `toff` of its 64-key tile
     int tkey[NL];
-    uint32_t toff[NL];
+    uint32_t toff[NL], tcol[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         const int idx = tid + i * kPfThreads;
-        const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
+        const int key = idx / CPR, col = (idx - key * CPR) ^ swz(key);
         tkey[i] = key;
-        toff[i] = (uint32_t)(((key % kPfKeys) * DH + oct * 8) * sizeof(uint16_t));
+        tcol[i] = (uint32_t)(col * 16);
+        toff[i] = (uint32_t)((key % kPfKeys) * DH * sizeof(uint16_t) + col * 16);
     }
-    auto fetch = [&](int kt) {
-        if (PAGE64) {
-            // one page lookup per tile, the same for every lane: the tile's first row is a scalar address and a load
-            // adds the thread's constant offset to it
+    typedef const void __attribute__((address_space(1)))* gptr_t;
+    typedef void __attribute__((address_space(3)))* lptr_t;
+    auto issue = [&](int kt, auto stage_c) {
+        uint16_t* const kdst = (decltype(stage_c)::value ? stage1 : stage0) + (tid & ~63) * 8;       // this wave's 1 KB of the first pass
+        uint16_t* const vdst = kdst + GROUPS * TILE;
+        // PAGE64 (pages of 64 tokens and more): a 64-key tile lies in one page; when the whole step lies inside the keys
+        // this tile may read, one page lookup per tile does, the same for every lane: the tile's first row is a scalar
+        // address and a load adds the thread's constant offset to it.
+        if (PAGE64 && kt >= first_key && kt + STEP - 1 <= last_key) {
             const char* krow[GROUPS];
             const char* vrow[GROUPS];
 #pragma unroll
             for (int t = 0; t < GROUPS; ++t) {
                 const int k0 = kt + kPfKeys * t;
-                const int k0c = (k0 <= last_key) ? k0 : last_key;     // a tile beyond the end is not loaded at all
-                const int pg = __builtin_amdgcn_readfirstlane(page_of(k0c));
+                const int pg = __builtin_amdgcn_readfirstlane(page_of(k0));
                 const size_t row = (size_t)pg * page_stride + (size_t)(k0 & page_mask) * DH;
                 krow[t] = reinterpret_cast<const char*>(kbase + row);
                 vrow[t] = reinterpret_cast<const char*>(vbase + row);
             }
 #pragma unroll
             for (int i = 0; i < NL; ++i) {
-                const int ka = kt + tkey[i];
-                kreg[i] = make_uint4(0, 0, 0, 0);
-                vreg[i] = make_uint4(0, 0, 0, 0);
-                if (ka <= last_key && ka >= first_key) {
-                    kreg[i] = *reinterpret_cast<const uint4*>(krow[(i * KPI) / kPfKeys] + toff[i]);
-                    vreg[i] = *reinterpret_cast<const uint4*>(vrow[(i * KPI) / kPfKeys] + toff[i]);
-                }
+                __builtin_amdgcn_global_load_lds((gptr_t)(krow[(i * KPI) / kPfKeys] + toff[i]), (lptr_t)(kdst + i * kPfThreads * 8), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(vrow[(i * KPI) / kPfKeys] + toff[i]), (lptr_t)(vdst + i * kPfThreads * 8), 16, 0, 0);
             }
             return;
         }
+        // Otherwise every load looks its page up.  A key outside what the tile may read (before the window's first key,
+        // beyond the last key) is replaced by the nearest one inside: its page may not be the request's any more, or not
+        // written yet; the mask drops its score, and the value it is multiplied with is a real one.
 #pragma unroll
         for (int i = 0; i < NL; ++i) {
-            const int idx = tid + i * kPfThreads;
-            const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
-            const int ka = kt + key;
-            kreg[i] = make_uint4(0, 0, 0, 0);
-            vreg[i] = make_uint4(0, 0, 0, 0);
-            if (ka <= last_key && ka >= first_key) {
-                const size_t off = (size_t)page_of(ka) * page_stride + (size_t)(ka & page_mask) * DH + oct * 8;
-                kreg[i] = *reinterpret_cast<const uint4*>(kbase + off);
-                vreg[i] = *reinterpret_cast<const uint4*>(vbase + off);
-            }
-        }
-    };
-    auto stash = [&]() {
-#pragma unroll
-        for (int i = 0; i < NL; ++i) {
-            const int idx = tid + i * kPfThreads;
-            const int key = idx / (DH / 8), oct = idx - key * (DH / 8);
-            *reinterpret_cast<uint4*>(&Ks_all[(key / kPfKeys) * KT + (key % kPfKeys) * KS + oct * 8]) = kreg[i];
-            *reinterpret_cast<uint4*>(&Vs_all[(key / kPfKeys) * VT + (key % kPfKeys) * VS + oct * 8]) = vreg[i];
+            int ka = kt + tkey[i];
+            ka = ka < first_key ? first_key : ka;
+            ka = ka > last_key ? last_key : ka;
+            const size_t off = ((size_t)page_of(ka) * page_stride + (size_t)(ka & page_mask) * DH) * sizeof(uint16_t) + tcol[i];
+            __builtin_amdgcn_global_load_lds((gptr_t)(reinterpret_cast<const char*>(kbase) + off), (lptr_t)(kdst + i * kPfThreads * 8), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(reinterpret_cast<const char*>(vbase) + off), (lptr_t)(vdst + i * kPfThreads * 8), 16, 0, 0);
         }
     };
 
-    const uint16_t* const Ks = Ks_all + grp * KT;
-    const uint16_t* const Vs = Vs_all + grp * VT;
-    fetch(kb_begin);
-    for (int kb = kb_begin; kb < kb_end; kb += STEP) {
-        __syncthreads();                                     // the previous step's readers are done
-        stash();
-        __syncthreads();
-        if (kb + STEP < kb_end) fetch(kb + STEP);            // in flight while this step is used
+    // where this lane reads its operands: K row lq (and 32 on), chunks 2 c + half; V rows 4 half + (l % 16) / 4 of a
+    // 16-key chunk (and 8 on), dims 32 dt + 16 (l / 16 % 2) + 4 (l % 4) ..+3
+    int koff[NC], voff[ND];
+    {
+        const int fq = swz(lq);
+#pragma unroll
+        for (int c = 0; c < NC; ++c) koff[c] = lq * DH + ((2 * c + half) ^ fq) * 8;
+        const int vrow = 4 * half + ((lane & 15) >> 2), fv = swz(vrow);
+#pragma unroll
+        for (int dt = 0; dt < ND; ++dt) voff[dt] = vrow * DH + ((4 * dt + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) ^ fv) * 8 + 4 * (lane & 1);
+    }
+
+    // one step: wait for its tiles, send for the next step's, use it
+    auto step = [&](int kb, auto stage_c) {
+        constexpr int S = decltype(stage_c)::value;
+        asm volatile("s_waitcnt vmcnt(0)" ::: "memory");     // this thread's loads of the step have reached LDS
+        __syncthreads();                                     // everybody's have, and the other stage's readers are done
+        if (kb + STEP < kb_end) issue(kb + STEP, std::integral_constant<int, 1 - S>{});      // in flight while this step is used
+        const uint16_t* const Ks = (S ? stage1 : stage0) + grp * TILE;
+        const uint16_t* const Vs = (S ? stage1 : stage0) + (GROUPS + grp) * TILE;
         const int kt = kb + kPfKeys * grp;                   // this group's key tile
-        if (!wave_ok || kt > wave_last) continue;            // nothing this wave may see
-        if (window > 0 && kt + kPfKeys - 1 < wave_first - window + 1) continue;
+        if (!wave_ok || kt > wave_last) return;              // nothing this wave may see
+        if (window > 0 && kt + kPfKeys - 1 < wave_first - window + 1) return;
 
         // ---- S^T = K Q^T : two tiles of 32 keys ----------------------------------
         v16f sacc[2];
@@ -236,11 +243,10 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
         for (int tt = 0; tt < 2; ++tt) {
 #pragma unroll
             for (int r = 0; r < 16; ++r) sacc[tt][r] = 0.f;
-            const uint16_t* kp = &Ks[(32 * tt + lq) * KS + 8 * half];
 #pragma unroll
             for (int c = 0; c < NC; ++c) {
                 Frag8 a;
-                a.u = *reinterpret_cast<const uint4*>(kp + 16 * c);
+                a.u = *reinterpret_cast<const uint4*>(Ks + 32 * tt * DH + koff[c]);
                 sacc[tt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, qf[c].v, sacc[tt], 0, 0, 0);
             }
         }
@@ -302,30 +308,38 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             for (int dt = 0; dt < ND; ++dt) {
                 // this lane's chunk: key 16 kc + 4 half + (l % 16) / 4 (and 8 keys on), dims 32 dt + 16 (l / 16 % 2) + 4 (l % 4) ..+3;
                 // what comes back is dim 32 dt + lq of keys 16 kc + 4 half + e (and 8 keys on), e = 0..3
-                const uint16_t* vp = &Vs[(16 * kc + 4 * half + ((lane & 15) >> 2)) * VS + 32 * dt + 16 * ((lane >> 4) & 1) + 4 * (lane & 3)];
+                const uint16_t* vp = Vs + 16 * kc * DH + voff[dt];
                 Frag8 a;
                 a.h[0] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)vp));
-                a.h[1] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)(vp + 8 * VS)));
+                a.h[1] = __builtin_bit_cast(uint2, __builtin_amdgcn_ds_read_tr16_b64_v4i16((tr_v4s __attribute__((address_space(3)))*)(vp + 8 * DH)));
                 oacc[dt] = __builtin_amdgcn_mfma_f32_32x32x16_bf16(a.v, b, oacc[dt], 0, 0, 0);
             }
         }
+    };
+    issue(kb_begin, std::integral_constant<int, 0>{});
+    for (int kb = kb_begin; kb < kb_end; kb += 2 * STEP) {
+        step(kb, std::integral_constant<int, 0>{});
+        if (kb + STEP < kb_end) step(kb + STEP, std::integral_constant<int, 1>{});
     }
 
     // ---- the odd-tile group hands its state to the even-tile group (same lane, same rows) ----------
     if (GROUPS == 2) {
     __syncthreads();                                         // every wave is done with the tiles
-    float* const mbuf = reinterpret_cast<float*>(tilebuf) + (size_t)(wave * 64 + lane) * MERGE_F;
+    // (the maximum, the sum and the first half of O^T's tiles through one stage's memory, the other half through the other's)
+    constexpr int H0 = ND / 2, F0 = 2 + 16 * H0, F1 = 16 * (ND - H0);
+    float* const mbuf0 = reinterpret_cast<float*>(stage0) + (size_t)(wave * 64 + lane) * F0;
+    float* const mbuf1 = reinterpret_cast<float*>(stage1) + (size_t)(wave * 64 + lane) * F1;
     if (grp == 1) {
-        mbuf[0] = m; mbuf[1] = l;
+        mbuf0[0] = m; mbuf0[1] = l;
 #pragma unroll
         for (int i = 0; i < ND; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) mbuf[2 + 16 * i + r] = oacc[i][r];
+            for (int r = 0; r < 16; ++r) (i < H0 ? mbuf0[2 + 16 * i + r] : mbuf1[16 * (i - H0) + r]) = oacc[i][r];
     }
     __syncthreads();
     if (grp == 1) return;
     {
-        const float m1 = mbuf[0], l1 = mbuf[1];
+        const float m1 = mbuf0[0], l1 = mbuf0[1];
         const float m_new = fmaxf(m, m1);
         const float mc = ((m_new == -INFINITY) ? 0.f : m_new) * scale_log2e;
         const float c0 = __builtin_amdgcn_exp2f(m * scale_log2e - mc), c1 = __builtin_amdgcn_exp2f(m1 * scale_log2e - mc);
@@ -333,7 +347,7 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
 #pragma unroll
         for (int i = 0; i < ND; ++i)
 #pragma unroll
-            for (int r = 0; r < 16; ++r) oacc[i][r] = oacc[i][r] * c0 + mbuf[2 + 16 * i + r] * c1;
+            for (int r = 0; r < 16; ++r) oacc[i][r] = oacc[i][r] * c0 + (i < H0 ? mbuf0[2 + 16 * i + r] : mbuf1[16 * (i - H0) + r]) * c1;
     }
     }
     // ---- a walk cut into parts: hand the state over, and the block that arrives last merges and writes ----------
