@@ -156,11 +156,13 @@ def test_rope_kv_write(dtype, nh, nkvh, dh, rot, page):
         _close(got[:, :nh][..., perm], adj, dtype)
 
 
-def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_width=0, groups=0, n_split=3, parts=None):
+def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_width=0, groups=0, n_split=3, parts=None,
+                    pages_given_back=False):
     """lens: list of (past, new) per request.  Returns (got, want) [T, nh*dh].  table_width pads
     the block tables with unused columns; groups is passed to the prompt-portion kernel; parts = (parts, part_len)
     cuts the prompt tiles' walks over the keys (the kernel is then launched twice: its arrival counters must come
-    back to zero)."""
+    back to zero).  pages_given_back (with a window): the block-table entries of pages that lie wholly before the
+    window of the step's first token name a page full of NaN, as if the manager had given them to someone else."""
     ops = _ops()
     g = torch.Generator().manual_seed(seed)
     scale = 1.0 / math.sqrt(dh)
@@ -173,6 +175,11 @@ def _attention_case(dtype, nh, nkvh, dh, page, lens, window, seed, impl, table_w
         v = torch.randn(t, nkvh, dh, generator=g).to(dtype)
         want.append(P.plain_attention(q, k, v, scale, past, window).reshape(new, nh * dh))
         kc, vc, bt = _paged(k, v, page, dtype, seed=seed + r)
+        if pages_given_back and window:
+            gone = max(0, past - window + 1) // page
+            spare = next(i for i in range(kc.shape[0]) if i not in set(bt.tolist()))      # an unused page: NaN throughout
+            bt = bt.clone()
+            bt[:gone] = spare
         kcs.append(kc); vcs.append(vc)
         tables.append(bt + page_base)
         page_base += kc.shape[0]
@@ -248,6 +255,29 @@ def test_attention_prefill_mfma(nh, nkvh, dh, page, window, groups):
     lens = [(0, 2), (0, 129), (130, 64), (64, 33), (15, 2), (257, 300), (5, 128)]
     got, want = _attention_case(torch.bfloat16, nh, nkvh, dh, page, lens, window, 13, "prefill", groups=groups)
     _close(got, want, torch.bfloat16, factor=3)
+
+
+@pytest.mark.parametrize("impl,dtype,groups,parts", [("prefill", torch.bfloat16, 1, None), ("prefill", torch.bfloat16, 2, None),
+                                                      ("prefill", torch.bfloat16, 1, (3, 1)), ("prefill", torch.float32, 0, None),
+                                                      ("generic", torch.bfloat16, 0, None), ("generic", torch.float32, 0, None)])
+@pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 2, 64, 16), (3, 3, 64, 64), (4, 1, 128, 32), (2, 2, 128, 128)])
+def test_attention_never_reads_pages_that_the_window_has_passed(impl, dtype, groups, parts, nh, nkvh, dh, page):
+    """The cache manager gives a page back as soon as a window has passed it, and someone else may write it: the
+    block-table entries before the window then name a page of NaN here, the rows of the last page beyond the last
+    key are NaN anyway, and nothing of either may reach the result (a NaN value times a probability of 0 is NaN)."""
+    lens = [(700, 140), (257, 300), (130, 64), (1000, 33), (90, 2), (5, 128)]
+    got, want = _attention_case(dtype, nh, nkvh, dh, page, lens, 100, 43, impl, groups=groups, parts=parts, pages_given_back=True)
+    assert bool(torch.isfinite(got.float()).all())
+    _close(got, want, dtype, factor=3)
+
+
+def test_attention_of_single_tokens_never_reads_pages_that_the_window_has_passed():
+    for dtype, nh, nkvh, dh, page, n_split in [(torch.bfloat16, 6, 6, 64, 16, 1), (torch.bfloat16, 8, 2, 128, 64, 3),
+                                                (torch.float32, 4, 2, 64, 32, 3), (torch.bfloat16, 16, 1, 64, 16, 2)]:
+        lens = [(700, 1), (99, 1), (100, 1), (1031, 1), (163, 1)]
+        got, want = _attention_case(dtype, nh, nkvh, dh, page, lens, 100, 44, "decode", n_split=n_split, pages_given_back=True)
+        assert bool(torch.isfinite(got.float()).all())
+        _close(got, want, dtype, factor=3)
 
 
 @pytest.mark.parametrize("nh,nkvh,dh,page", [(6, 6, 64, 16), (6, 2, 64, 64), (3, 1, 64, 32), (4, 2, 128, 16), (4, 4, 128, 64)])
