@@ -74,10 +74,13 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     static_assert(GROUPS == 1 || sizeof(uint16_t) * STAGE >= sizeof(float) * 256 * (2 + (ND / 2) * 16), "each half of the merge buffer fits in a stage");
     // Two stages: the loads of the next step write one while the other is read.  They go from memory straight into LDS
     // (global_load_lds_dwordx4: lane i of a wave writes 16 bytes at the wave's base + 16 i, no registers, no store
-    // instructions), so rows cannot be padded; instead the 16-byte chunks of row r sit at position (chunk ^ swz(r)), which a
-    // lane arranges by fetching the chunk that belongs where it writes.  With swz(r) = 2 (r % 4) + (r / 4) % 2 the 16-byte
-    // reads of 8 consecutive rows (K operand) and the transposing 8-byte reads of 4 consecutive rows x 32 bytes (V operand)
-    // each cover all banks once.
+    // instructions), so rows cannot be padded; instead the 16-byte chunks of row r sit at position (chunk ^ f(r)), which a
+    // lane arranges by fetching the chunk that belongs where it writes.  The LDS has 64 banks of 4 bytes: a 16-byte read of
+    // a wave is conflict-free when 16 consecutive rows fall on 16 different 16-byte slots of the 256 bytes, so for the K
+    // operand f(r) = r / 2 % 8 with rows of 128 bytes and r % 16 with rows of 256; the transposing 8-byte reads of the V
+    // operand (4 rows x 32 bytes per 16 lanes) want f(r) = 2 (r % 4) + (r / 4) % 2.  Measured alone, cycles per read
+    // instruction with four waves reading: K 20 (32 with f = r % 8, 22 with rows padded to 144 bytes, 128 with neither),
+    // V 20 (19 with rows padded to 160 bytes).
     // (Two arrays, and the stage a compile-time constant wherever they are used: the compiler then knows that a load
     // in flight into one does not touch what is read from the other, and does not wait for it before every LDS read.)
     __shared__ __attribute__((aligned(16))) uint16_t stage0[STAGE];
@@ -159,19 +162,22 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     const size_t page_stride = (size_t)nkvh * head_stride;
 
     // What a thread loads in a step never changes: LDS chunk tid + i * threads of the step's K (and V) tiles, that is key
-    // `tkey` of the step's keys at chunk position idx % CPR, which holds the row's chunk `pos ^ swz(key)`.
-    auto swz = [](int row) -> int { return ((row & 3) << 1) | ((row >> 2) & 1); };
+    // `tkey` of the step's keys at chunk position idx % CPR, which holds the row's chunk `pos ^ f(key)`.
+    auto swz_k = [](int row) -> int { return DH == 64 ? (row >> 1) & 7 : row & 15; };
+    auto swz_v = [](int row) -> int { return ((row & 3) << 1) | ((row >> 2) & 1); };
     constexpr int KPI = kPfThreads / CPR;                     // keys one pass of loads covers (<= 64)
     static_assert(KPI <= kPfKeys && kPfKeys % KPI == 0, "a pass of loads stays inside a tile");
     int tkey[NL];
-    uint32_t toff[NL], tcol[NL];
+    uint32_t toffk[NL], toffv[NL], tcolk[NL], tcolv[NL];
 #pragma unroll
     for (int i = 0; i < NL; ++i) {
         const int idx = tid + i * kPfThreads;
-        const int key = idx / CPR, col = (idx - key * CPR) ^ swz(key);
+        const int key = idx / CPR, colk = (idx - key * CPR) ^ swz_k(key), colv = (idx - key * CPR) ^ swz_v(key);
         tkey[i] = key;
-        tcol[i] = (uint32_t)(col * 16);
-        toff[i] = (uint32_t)((key % kPfKeys) * DH * sizeof(uint16_t) + col * 16);
+        tcolk[i] = (uint32_t)(colk * 16);
+        tcolv[i] = (uint32_t)(colv * 16);
+        toffk[i] = (uint32_t)((key % kPfKeys) * DH * sizeof(uint16_t) + colk * 16);
+        toffv[i] = (uint32_t)((key % kPfKeys) * DH * sizeof(uint16_t) + colv * 16);
     }
     typedef const void __attribute__((address_space(1)))* gptr_t;
     typedef void __attribute__((address_space(3)))* lptr_t;
@@ -194,8 +200,8 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             }
 #pragma unroll
             for (int i = 0; i < NL; ++i) {
-                __builtin_amdgcn_global_load_lds((gptr_t)(krow[(i * KPI) / kPfKeys] + toff[i]), (lptr_t)(kdst + i * kPfThreads * 8), 16, 0, 0);
-                __builtin_amdgcn_global_load_lds((gptr_t)(vrow[(i * KPI) / kPfKeys] + toff[i]), (lptr_t)(vdst + i * kPfThreads * 8), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(krow[(i * KPI) / kPfKeys] + toffk[i]), (lptr_t)(kdst + i * kPfThreads * 8), 16, 0, 0);
+                __builtin_amdgcn_global_load_lds((gptr_t)(vrow[(i * KPI) / kPfKeys] + toffv[i]), (lptr_t)(vdst + i * kPfThreads * 8), 16, 0, 0);
             }
             return;
         }
@@ -207,9 +213,9 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
             int ka = kt + tkey[i];
             ka = ka < first_key ? first_key : ka;
             ka = ka > last_key ? last_key : ka;
-            const size_t off = ((size_t)page_of(ka) * page_stride + (size_t)(ka & page_mask) * DH) * sizeof(uint16_t) + tcol[i];
-            __builtin_amdgcn_global_load_lds((gptr_t)(reinterpret_cast<const char*>(kbase) + off), (lptr_t)(kdst + i * kPfThreads * 8), 16, 0, 0);
-            __builtin_amdgcn_global_load_lds((gptr_t)(reinterpret_cast<const char*>(vbase) + off), (lptr_t)(vdst + i * kPfThreads * 8), 16, 0, 0);
+            const size_t off = ((size_t)page_of(ka) * page_stride + (size_t)(ka & page_mask) * DH) * sizeof(uint16_t);
+            __builtin_amdgcn_global_load_lds((gptr_t)(reinterpret_cast<const char*>(kbase) + off + tcolk[i]), (lptr_t)(kdst + i * kPfThreads * 8), 16, 0, 0);
+            __builtin_amdgcn_global_load_lds((gptr_t)(reinterpret_cast<const char*>(vbase) + off + tcolv[i]), (lptr_t)(vdst + i * kPfThreads * 8), 16, 0, 0);
         }
     };
 
@@ -217,10 +223,10 @@ attn_prefill_mfma_kernel(const uint16_t* __restrict__ q, int q_stride, uint16_t*
     // 16-key chunk (and 8 on), dims 32 dt + 16 (l / 16 % 2) + 4 (l % 4) ..+3
     int koff[NC], voff[ND];
     {
-        const int fq = swz(lq);
+        const int fq = swz_k(lq);
 #pragma unroll
         for (int c = 0; c < NC; ++c) koff[c] = lq * DH + ((2 * c + half) ^ fq) * 8;
-        const int vrow = 4 * half + ((lane & 15) >> 2), fv = swz(vrow);
+        const int vrow = 4 * half + ((lane & 15) >> 2), fv = swz_v(vrow);
 #pragma unroll
         for (int dt = 0; dt < ND; ++dt) voff[dt] = vrow * DH + ((4 * dt + 2 * ((lane >> 4) & 1) + ((lane & 3) >> 1)) ^ fv) * 8 + 4 * (lane & 1);
     }
