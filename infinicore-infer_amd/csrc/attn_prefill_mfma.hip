@@ -431,27 +431,46 @@ IC_EXPORT long long ic_attn_prefill_scratch_floats(int n_tiles, int nh, int dh, 
 }
 
 // How to cut the walks of a step whose longest query tile sees `max_keys` keys: parts per tile (1: no cut) and key tiles
-// per part.  From a sweep over 16..48 heads of 64 and 32..40 of 128, prompts of 300..4,096 tokens and portions of 256..1,024
-// after 1,024..3,584 tokens, against one and two wave groups:
-//  * parts pay when walks are long (24 key tiles and more) and blocks are few: as many parts as keep about 4.5 blocks a compute
-//    unit at head size 64 and 2 at head size 128 (what stays resident there), at most 4, each of 6 key tiles or more;
+// per part.  From sweeps over 16..48 heads of 64 and 32..40 of 128, prompts of 300..4,096 tokens and portions of 256..1,024
+// after 256..3,584 tokens, against one and two wave groups:
+//  * with many blocks, parts pay when walks are long (24 key tiles and more): as many parts as keep about 4.5 blocks a compute
+//    unit at head size 64 and 2 at head size 128 (what stays resident there), at most 4, each of 6 key tiles or more; two
+//    parts do no better than two wave groups where those run (up to 2 blocks a unit), so they keep that case;
+//  * with few blocks (a portion or two beside decoded tokens) shorter walks are cut too: head size 64, up to half a block a
+//    unit, from 12 key tiles on into 3 parts (4 from 20 key tiles on when four parts of every block still fit the units at once), and up to 1.25 blocks a unit
+//    from 20 key tiles on into 3; head size 128, up to half a block a unit, walks of 8..23 key tiles into 2 parts, and up to a
+//    quarter block a unit from 16 key tiles on into 4.  Against two wave groups, portions of 512 tokens after 512..768:
+//    24:8 x 64 (96 blocks) 17.6 -> 14.7 and 20.0 -> 17.0 us, 32:2 x 128 (128 blocks) 25.9 -> 22.0 and 29.8 -> 25.1; 256
+//    tokens after 1,024: 19.8 -> 13.9 and 29.2 -> 19.9;
 //  * portions after a long past gain most (16 heads, 512 tokens after 3,584: 54 -> 26 us; 36 heads: 54 -> 41; 32:2 x 128: 83 -> 52),
-//    whole prompts little (36 heads, 2,048 tokens: 43 -> 41 us) or nothing;
-//  * two parts do no better than two wave groups where those run (up to 2 blocks a unit), so they keep that case.
+//    whole prompts little (36 heads, 2,048 tokens: 43 -> 41 us) or nothing.
 IC_EXPORT int ic_attn_prefill_parts(int n_tiles, int nh, int dh, int max_keys, int compute_units, int* part_len) {
     const int longest = (max_keys + kPfKeys - 1) / kPfKeys;
-    const long long blocks = (long long)n_tiles * nh;
+    const long long blocks = (long long)n_tiles * nh, cu = compute_units;
     int len = longest > 0 ? longest : 1, parts = 1;
-    if (compute_units > 0 && blocks > 0 && blocks <= kPfCounters && longest >= 24 && (dh == 64 || dh == 128)) {
-        const long long room = dh == 64 ? 9LL * compute_units / 2 : 2LL * compute_units;
-        long long p = room / blocks;
-        p = p > 4 ? 4 : p;
-        p = p > longest / 6 ? longest / 6 : p;
-        if (p == 2 && blocks <= 2LL * compute_units) p = 1;
+    if (compute_units > 0 && blocks > 0 && blocks <= kPfCounters && (dh == 64 || dh == 128)) {
+        long long p = 1;
+        int least = 6;                                      // key tiles a part has at least
+        bool few = false;
+        if (dh == 64) {
+            if (2 * blocks <= cu && longest >= 12) { p = (4 * blocks <= cu && longest >= 20) ? 4 : 3; few = true; }
+            else if (4 * blocks <= 5 * cu && longest >= 20) { p = 3; few = true; }
+        } else {
+            if (4 * blocks <= cu && longest >= 16) { p = 4; few = true; }
+            else if (2 * blocks <= cu && longest >= 8 && longest < 24) { p = 2; few = true; }
+        }
+        if (few) least = 4;
+        else if (longest >= 24) {
+            const long long room = dh == 64 ? 9LL * cu / 2 : 2LL * cu;
+            p = room / blocks;
+            p = p > 4 ? 4 : p;
+            if (p == 2 && blocks <= 2LL * cu) p = 1;
+        }
+        p = p > longest / least ? longest / least : p;
         if (p >= 2) {
             parts = (int)p;
             len = (longest + parts - 1) / parts;
-            len = len < 6 ? 6 : len;
+            len = len < least ? least : len;
         }
     }
     if (part_len) *part_len = len;

@@ -304,7 +304,12 @@ def test_attention_prefill_with_the_walk_over_the_keys_cut_into_parts(nh, nkvh, 
 def test_attention_prefill_parts_rule_and_its_refusals():
     ops = _ops()
     assert ops.attention_prefill_parts(16, 36, 64, 2048, 256) == (2, 16)         # the benchmark's prompt: 576 blocks of 32 key tiles
-    assert ops.attention_prefill_parts(4, 36, 64, 2048, 256)[0] == 4             # a portion of 512 after 1,536
+    assert ops.attention_prefill_parts(4, 36, 64, 2048, 256) == (3, 11)          # a portion of 512 after 1,536: few blocks, three parts
+    assert ops.attention_prefill_parts(4, 24, 64, 1024, 256) == (3, 6)           # few blocks: walks of 12 key tiles and more are cut
+    assert ops.attention_prefill_parts(2, 24, 64, 1280, 256) == (4, 5)           # very few blocks and 20 key tiles: four parts
+    assert ops.attention_prefill_parts(4, 24, 64, 704, 256)[0] == 1              # 11 key tiles: left whole
+    assert ops.attention_prefill_parts(4, 32, 128, 1024, 256) == (2, 8) and ops.attention_prefill_parts(2, 32, 128, 1280, 256) == (4, 5)
+    assert ops.attention_prefill_parts(8, 32, 128, 1024, 256)[0] == 1            # a block a unit at head size 128: two wave groups do it
     assert ops.attention_prefill_parts(4, 36, 64, 1024, 256)[0] == 1             # short walks are left whole
     assert ops.attention_prefill_parts(32, 36, 64, 4096, 256)[0] == 1            # many blocks too
     assert ops.attention_prefill_parts(16, 32, 128, 2048, 256)[0] == 1 and ops.attention_prefill_parts(4, 40, 128, 4096, 256)[0] == 3
