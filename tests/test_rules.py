@@ -82,3 +82,28 @@ def test_attention_kernels_of_a_step():
     assert ops.attention_decode_splits(8, 36, 36, 64, 2, 0, 256, 0, 256) == 1
     assert ops.attention_decode_splits(1, 36, 36, 64, 2, 0, 16384, 0, 256) > 4
     assert ops.attention_decode_splits(64, 36, 36, 64, 2, 0, 2560, 0, 256) == 1
+
+
+def test_cut_walks_of_prompt_tiles():
+    """How a step's prompt tiles are cut: (tiles, heads, head size, keys the longest tile sees, compute units) -> (parts, key
+    tiles a part)."""
+    ops = _ops()
+    parts = ops.attention_prefill_parts
+    assert parts(16, 36, 64, 2048, 256) == (2, 16)          # the benchmark's prompt: 576 blocks of 32 key tiles
+    assert parts(32, 36, 64, 4096, 256)[0] == 1             # many blocks: left whole
+    assert parts(16, 32, 128, 2048, 256)[0] == 1            # two blocks a unit at head size 128: two wave groups do it
+    assert parts(4, 40, 128, 4096, 256) == (3, 22)
+    # few blocks (a portion or two beside decoded tokens): shorter walks are cut too
+    assert parts(4, 36, 64, 2048, 256) == (3, 11) and parts(4, 24, 64, 1024, 256) == (3, 6) and parts(2, 24, 64, 1280, 256) == (4, 5)
+    assert parts(4, 24, 64, 704, 256)[0] == 1 and parts(4, 36, 64, 1024, 256)[0] == 1
+    assert parts(4, 32, 128, 1024, 256) == (2, 8) and parts(2, 32, 128, 1280, 256) == (4, 5) and parts(8, 32, 128, 1024, 256)[0] == 1
+    # a part never has fewer key tiles than the rule's least, and the parts cover the walk
+    for tiles in (1, 2, 4, 8, 16):
+        for heads, dh in ((8, 64), (24, 64), (36, 64), (32, 128), (2, 128)):
+            for keys in range(64, 8200, 448):
+                p, n = parts(tiles, heads, dh, keys, 256)
+                longest = (keys + 63) // 64
+                assert 1 <= p <= 4 and p * n >= longest and (p == 1 or n >= 4)
+    # the scratch memory the parts need
+    assert ops.attention_prefill_scratch_floats(4, 36, 64, 4) == 4 * 36 * 4 * 256 * 34 and ops.attention_prefill_scratch_floats(4, 36, 64, 1) == 0
+
