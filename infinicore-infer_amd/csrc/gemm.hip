@@ -97,8 +97,13 @@ __device__ __forceinline__ void spread_token_operand(const v4s* glo, const v4s* 
 // LINES (K a multiple of 64, aligned operands): the weights come in whole cache lines, a wave's load covering 8 rows x
 // 128 bytes (two k-steps), with the non-temporal hint: a kernel that only streams a weight matrix so takes 9.4 us for
 // the 2B shape's 53 MB gate/up matrix where loads in operand layout (16 rows x 64 bytes) take 15.6.  What a load
-// brings is not in operand layout, so each wave passes it through 2.3 KB of LDS of its own (rows 144 bytes apart: the
-// 16 rows of an operand read then fall into different banks) on its way to the matrix cores.
+// brings is not in operand layout, so each wave passes it through LDS of its own on its way to the matrix cores.  In the
+// kernel below the loads write it there themselves (global_load_lds_dwordx4: lane l puts 16 bytes at the tile's half +
+// 16 l, no registers and no LDS store instructions, which take 13 cycles per KB and unit where reads take 6): rows of
+// 128 bytes without padding, chunk c of row r at position c ^ (r / 2 % 8), which each lane arranges by what it fetches, so
+// that the 16-byte operand reads of 16 rows cover the 64 banks once; a tile of 2 KB per pair of k-steps in flight and
+// 16-row tile.  2B shape, recorded steps, against registers + ds_write: batch 1 1.90 -> 1.88 ms, batch 8 2.92 -> 2.89.
+// The kernel for very many weight rows further down still stores from registers, into rows 144 bytes apart.
 constexpr int kLineRowBytes = 144;
 template <typename TC, int NT, int MT, int WPB, int UNROLL, bool ALIGNED, int EPI, bool OWN_K = false, int AG = 1, bool LINES = false>
 __global__ void __launch_bounds__(WPB * 64)
@@ -110,7 +115,8 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     constexpr int PV = kMaxSumParts / (WPB * 4);             // column-block sums a thread fetches
     static_assert(!LINES || (ALIGNED && UNROLL % 2 == 0), "whole-line weight loads take k-steps in pairs");
     // the waves' partial sums after the loop; while the loop runs the same memory passes the weights on (LINES)
-    constexpr int kRedBytes = (WPB - 1) * NT * MT * 64 * 4 * 4, kLineBytes = LINES ? WPB * 16 * kLineRowBytes : 0;
+    constexpr int kWaveLineBytes = (UNROLL / 2 > 0 ? UNROLL / 2 : 1) * NT * 2048;      // a wave's tiles of an iteration: 16 rows x 128 bytes each
+    constexpr int kRedBytes = (WPB - 1) * NT * MT * 64 * 4 * 4, kLineBytes = LINES ? WPB * kWaveLineBytes : 0;
     __shared__ __attribute__((aligned(16))) unsigned char red_mem[kRedBytes > kLineBytes ? kRedBytes : kLineBytes];
     float (*red)[NT * MT][64][4] = reinterpret_cast<float (*)[NT * MT][64][4]>(red_mem);
     __shared__ float ssum[WPB * 4][16];
@@ -169,11 +175,11 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
 #pragma unroll
             for (int h = 0; h < 2; ++h) {
                 const int row = base + 8 * h + (lane >> 3);
-                wp8[nt][h] = W + (size_t)(row < lim ? row : lim - 1) * ldw + 8 * (lane & 7);
+                wp8[nt][h] = W + (size_t)(row < lim ? row : lim - 1) * ldw + 8 * ((lane & 7) ^ (((8 * h + (lane >> 3)) >> 1) & 7));
             }
         }
     }
-    unsigned char* const line_buf = red_mem + (LINES ? wave * 16 * kLineRowBytes : 0);
+    unsigned char* const line_buf = red_mem + (LINES ? wave * kWaveLineBytes : 0);
     const uint16_t* ap[MT];
 #pragma unroll
     for (int mt = 0; mt < MT; ++mt) {
@@ -221,17 +227,23 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
     constexpr int it_stride = PAIR_DEAL ? WPB * (UNROLL / 2) : s_stride * UNROLL;
     for (int s0 = s_begin; s0 < it_end; s0 += it_stride) {
         v4s wlo[LINES ? 1 : UNROLL][NT], whi[LINES ? 1 : UNROLL][NT], alo[UNROLL][MT], ahi[UNROLL][MT];
-        uint4 wline[LINES ? UNROLL / 2 : 1][NT][2];
         if constexpr (LINES) {
+            // straight into this wave's LDS (lane l writes 16 bytes at the tile's half + 16 l: rows of 128 bytes without
+            // padding, their chunks swizzled by the choice of what each lane fetches), with the non-temporal hint
+            typedef const void __attribute__((address_space(1)))* gptr_t;
+            typedef void __attribute__((address_space(3)))* lptr_t;
 #pragma unroll
             for (int j = 0; j < UNROLL / 2; ++j) {
                 const int st = step_at(s0, 2 * j);
-                const bool ok = st < s_end;                  // (both steps of the pair exist, or neither)
+                // a pair beyond the end loads the first one again and is multiplied with zeros: the loads stay without a
+                // condition (measured: skipping them, with the wait that a branch then needs written out, was 1 % slower at
+                // batch 8; and the compiler's own wait for loads into LDS does not survive a branch)
+                const int stc = st < s_end ? st : 0;
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt)
 #pragma unroll
                     for (int h = 0; h < 2; ++h)
-                        wline[j][nt][h] = ok ? load_stream16(wp8[nt][h] + 32 * st) : uint4{0, 0, 0, 0};
+                        __builtin_amdgcn_global_load_lds((gptr_t)(wp8[nt][h] + 32 * stc), (lptr_t)(line_buf + (j * NT + nt) * 2048 + 1024 * h), 16, 0, 2);
             }
         } else {
 #pragma unroll
@@ -280,19 +292,15 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
         typedef __bf16 v8b __attribute__((ext_vector_type(8)));
         if constexpr (LINES) {
 #pragma unroll
-            for (int j = 0; j < UNROLL / 2; ++j)
+            for (int j = 0; j < UNROLL / 2; ++j) {
 #pragma unroll
                 for (int nt = 0; nt < NT; ++nt) {
                     // through this wave's LDS: in as rows of 128 bytes, out as the operands of the pair's two k-steps
                     // (row r, bytes 16 kq .. of the first half and of the second).  LDS serves a wave's requests in order.
-#pragma unroll
-                    for (int h = 0; h < 2; ++h)
-                        *reinterpret_cast<uint4*>(line_buf + (8 * h + (lane >> 3)) * kLineRowBytes + 16 * (lane & 7)) = wline[j][nt][h];
-                    __builtin_amdgcn_wave_barrier();
                     uint4 w2[2];
 #pragma unroll
-                    for (int e = 0; e < 2; ++e) w2[e] = *reinterpret_cast<const uint4*>(line_buf + r * kLineRowBytes + 16 * (4 * e + kq));
-                    __builtin_amdgcn_wave_barrier();
+                    for (int e = 0; e < 2; ++e)
+                        w2[e] = *reinterpret_cast<const uint4*>(line_buf + (j * NT + nt) * 2048 + r * 128 + 16 * ((4 * e + kq) ^ ((r >> 1) & 7)));
 #pragma unroll
                     for (int e = 0; e < 2; ++e)
 #pragma unroll
@@ -302,6 +310,7 @@ gemm_nt_bf16_kernel(const uint16_t* __restrict__ A, const uint16_t* __restrict__
                                                                                   acc[nt][mt], 0, 0, 0);
                         }
                 }
+            }
         } else {
 #pragma unroll
         for (int u = 0; u < UNROLL; ++u)
